@@ -1,0 +1,168 @@
+/*
+ * TEST INFRASTRUCTURE ONLY - drives the reference's own compiled CPU attention.
+ *
+ * Built only where the reference checkout exists (see oracle/Makefile); it
+ * includes the reference headers by path and links the reference's own
+ * Matrix / Softmax / RotaryEmbedding / CausalSelfAttention / UniformInit
+ * objects.  No reference source is copied into this repository.
+ *
+ * The reference layer (Layers/CausalSelfAttention.hpp:44-88) only accepts an
+ * embedding matrix X and projection weights.  To feed it raw Q, K, V the
+ * driver stacks X = [Q; K; V] and uses 0/1 selection matrices for W_q, W_k,
+ * W_v (exact in fp32), W_o = identity, and overwrites the public RoPE tables
+ * with cos = 1, sin = 0 (RotaryEmbedding.hpp:20-21), so that
+ *   cache.attended       = O
+ *   cache.scores[h]      = scaled, masked scores  (-> LSE)
+ *   cache.queryGradient  = dQ, cache.keyGradient = dK, cache.valueGradient = dV
+ * come straight out of the reference's forward / backward.
+ * The layer always uses scale = 1/sqrt(headDim) and the causal mask.
+ */
+#include "NeuralNet/Activations/Softmax.hpp"
+#include "NeuralNet/Layers/CausalSelfAttention.hpp"
+#include "NeuralNet/Layers/RotaryEmbedding.hpp"
+#include "NeuralNet/Math/Matrix.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstddef>
+#include <exception>
+#include <vector>
+
+namespace {
+
+Matrix selection(int rows, int cols, int colOffset) {
+    Matrix w(static_cast<size_t>(rows), static_cast<size_t>(cols), 0.0f);
+    for (int r = 0; r < rows; ++r) w.at(static_cast<size_t>(r), static_cast<size_t>(colOffset + r)) = 1.0f;
+    return w;
+}
+
+void runLayer(const float* q, const float* k, const float* v, float* out, float* lse, const float* dOut, float* dq,
+              float* dk, float* dv, int qHeads, int kvHeads, int d, size_t stride, size_t col0, int t, int qHead0,
+              int kvHead0, bool accumulateKv) {
+    const int qRows = qHeads * d;
+    const int kvRows = kvHeads * d;
+    const int embed = qRows + 2 * kvRows;
+
+    RotaryEmbedding rope(d, t);
+    std::fill(rope.cosTable.begin(), rope.cosTable.end(), 1.0f);
+    std::fill(rope.sinTable.begin(), rope.sinTable.end(), 0.0f);
+
+    CausalSelfAttention layer(selection(qRows, embed, 0), selection(kvRows, embed, qRows),
+                              selection(kvRows, embed, qRows + kvRows), selection(qRows, qRows, 0), rope, qHeads, t, 0,
+                              kvHeads);
+
+    Matrix x(static_cast<size_t>(embed), static_cast<size_t>(t), 0.0f);
+    for (int r = 0; r < qRows; ++r)
+        for (int c = 0; c < t; ++c) x.at(r, c) = q[(static_cast<size_t>(qHead0) * d + r) * stride + col0 + c];
+    for (int r = 0; r < kvRows; ++r)
+        for (int c = 0; c < t; ++c) {
+            x.at(qRows + r, c) = k[(static_cast<size_t>(kvHead0) * d + r) * stride + col0 + c];
+            x.at(qRows + kvRows + r, c) = v[(static_cast<size_t>(kvHead0) * d + r) * stride + col0 + c];
+        }
+
+    CausalSelfAttentionCache cache;
+    layer.forward(x, cache);
+    for (int r = 0; r < qRows; ++r)
+        for (int c = 0; c < t; ++c) out[(static_cast<size_t>(qHead0) * d + r) * stride + col0 + c] = cache.attended.at(r, c);
+
+    if (lse) {
+        for (int h = 0; h < qHeads; ++h) {
+            const Matrix& s = cache.scores[static_cast<size_t>(h)];
+            for (int query = 0; query < t; ++query) {
+                float top = s.at(0, query);
+                for (int key = 1; key < t; ++key) top = std::max(top, s.at(key, query));
+                double total = 0.0;
+                for (int key = 0; key < t; ++key) total += std::exp(static_cast<double>(s.at(key, query)) - static_cast<double>(top));
+                lse[static_cast<size_t>(qHead0 + h) * stride + col0 + query] = static_cast<float>(top + std::log(total));
+            }
+        }
+    }
+    if (!dOut) return;
+
+    Matrix g(static_cast<size_t>(qRows), static_cast<size_t>(t), 0.0f);
+    for (int r = 0; r < qRows; ++r)
+        for (int c = 0; c < t; ++c) g.at(r, c) = dOut[(static_cast<size_t>(qHead0) * d + r) * stride + col0 + c];
+    Matrix gwq, gwk, gwv, gwo;
+    layer.backward(g, cache, gwq, gwk, gwv, gwo);
+    for (int r = 0; r < qRows; ++r)
+        for (int c = 0; c < t; ++c)
+            dq[(static_cast<size_t>(qHead0) * d + r) * stride + col0 + c] = cache.queryGradient.at(r, c);
+    for (int r = 0; r < kvRows; ++r)
+        for (int c = 0; c < t; ++c) {
+            const size_t idx = (static_cast<size_t>(kvHead0) * d + r) * stride + col0 + c;
+            if (accumulateKv) {
+                dk[idx] += cache.keyGradient.at(r, c);
+                dv[idx] += cache.valueGradient.at(r, c);
+            } else {
+                dk[idx] = cache.keyGradient.at(r, c);
+                dv[idx] = cache.valueGradient.at(r, c);
+            }
+        }
+}
+
+}  // namespace
+
+/*
+ * Same argument meaning as sentinel_oracle_attention; `scale` must equal
+ * 1/sqrt(headDim) and causal must be 1 (the layer has no other mode).
+ * perHead = 0: one layer call per pack with all heads (native GQA inside the layer).
+ * perHead = 1: one single-head layer call per (pack, query head) to bound memory;
+ *              grouped dK / dV are added in increasing query-head order like
+ *              addHeadInto (Layers/CausalSelfAttention.cpp:187-193).
+ */
+extern "C" int sentinel_ref_attention(const float* q, const float* k, const float* v, float* out, float* lse,
+                                      const float* d_out, float* dq, float* dk, float* dv, int qHeads, int kvHeads,
+                                      int headDim, int strideColumns, int colStart, int seqLen, int packCount, int perHead) {
+    try {
+        if (qHeads <= 0 || kvHeads <= 0 || qHeads % kvHeads != 0) return -1;
+        const size_t stride = static_cast<size_t>(strideColumns);
+        for (int pack = 0; pack < packCount; ++pack) {
+            const size_t col0 = static_cast<size_t>(colStart) + static_cast<size_t>(pack) * seqLen;
+            if (!perHead) {
+                runLayer(q, k, v, out, lse, d_out, dq, dk, dv, qHeads, kvHeads, headDim, stride, col0, seqLen, 0, 0, false);
+                continue;
+            }
+            const int group = qHeads / kvHeads;
+            if (d_out)
+                for (int r = 0; r < kvHeads * headDim; ++r)
+                    for (int c = 0; c < seqLen; ++c) {
+                        dk[static_cast<size_t>(r) * stride + col0 + c] = 0.0f;
+                        dv[static_cast<size_t>(r) * stride + col0 + c] = 0.0f;
+                    }
+            for (int h = 0; h < qHeads; ++h)
+                runLayer(q, k, v, out, lse, d_out, dq, dk, dv, 1, 1, headDim, stride, col0, seqLen, h, h / group, true);
+        }
+        return 0;
+    } catch (const std::exception&) {
+        return -2;
+    }
+}
+
+extern "C" int sentinel_ref_gemm(const float* a, int aRows, int aCols, const float* b, int bRows, int bCols, float* c,
+                                 int transposeA, int transposeB) {
+    try {
+        Matrix left(static_cast<size_t>(aRows), static_cast<size_t>(aCols));
+        Matrix right(static_cast<size_t>(bRows), static_cast<size_t>(bCols));
+        std::copy(a, a + left.data.size(), left.data.begin());
+        std::copy(b, b + right.data.size(), right.data.begin());
+        Matrix result;
+        Matrix::gemm(left, right, result, transposeA != 0, transposeB != 0);
+        std::copy(result.data.begin(), result.data.end(), c);
+        return 0;
+    } catch (const std::exception&) {
+        return -2;
+    }
+}
+
+extern "C" int sentinel_ref_softmax_columns(const float* logits, float* out, int rows, int cols) {
+    try {
+        Matrix in(static_cast<size_t>(rows), static_cast<size_t>(cols));
+        std::copy(logits, logits + in.data.size(), in.data.begin());
+        Matrix result;
+        Softmax::applyInto(in, result);
+        std::copy(result.data.begin(), result.data.end(), out);
+        return 0;
+    } catch (const std::exception&) {
+        return -2;
+    }
+}

@@ -1,0 +1,340 @@
+/*
+ * TEST INFRASTRUCTURE ONLY - CPU oracle for Sentinel's causal attention.
+ *
+ * Restates, in plain C++ on raw arrays, the arithmetic of the reference's host
+ * attention path so that fp32 results carry the reference's own summation
+ * order.  The shipped library never links or calls this file; only tests/,
+ * __graft_entry__.smoke() and bench.py's cpu_baseline leg may use it.
+ *
+ * Reference sources followed (paths relative to the reference checkout):
+ *   sentinel/NeuralNet/Math/Matrix.cpp:11-72,106-148      blocked gemm, transposed packing, OpenMP rule
+ *   sentinel/NeuralNet/Activations/Softmax.cpp:10-44       column softmax
+ *   sentinel/NeuralNet/Layers/CausalSelfAttention.cpp:90-100   GQA head map, mask rule
+ *   sentinel/NeuralNet/Layers/CausalSelfAttention.cpp:122-126  scores = K^T Q, scale, mask
+ *   sentinel/NeuralNet/Layers/CausalSelfAttention.cpp:150-152  attended = V P
+ *   sentinel/NeuralNet/Layers/CausalSelfAttention.cpp:195-210  softmax backward
+ *   sentinel/NeuralNet/Layers/CausalSelfAttention.cpp:232-254  per-head forward
+ *   sentinel/NeuralNet/Layers/CausalSelfAttention.cpp:279-353  per-head backward (dense branch)
+ *   sentinel/NeuralNet/Cuda/CudaFlashAttention.cu:1260-1264    LSE = max + ln(sum)
+ *   sentinel/NeuralNet/Cuda/CudaFlashAttention.cu:576-596      D = rowsum(O * dO)
+ *
+ * How each function is pinned (see tests/test_oracle_*.py):
+ *   gemm, softmax, forward, backward : bit-compared with the reference's own
+ *       compiled CPU sources (oracle/_ref) on committed fixtures, and checked
+ *       against float64 brute force, closed forms (Q = 0, constant V, first
+ *       query) and central finite differences.
+ *   lse, delta : no CPU counterpart in the reference (device-only quantities);
+ *       pinned by their definitions in float64 and by closed forms.
+ *   causal = 0 : device-API flag with no CPU counterpart; pinned by float64
+ *       brute force only.
+ *
+ * Heads are processed one at a time (forward immediately followed by that
+ * head's backward) instead of caching every head's T x T probabilities as the
+ * reference layer does; heads are independent, and grouped K/V gradients are
+ * still added in increasing query-head order, so results are identical while
+ * memory stays at a few T x T matrices.
+ */
+#include "sentinel_attention_oracle.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstddef>
+#include <cstring>
+#include <vector>
+
+#if defined(_OPENMP)
+#include <omp.h>
+#endif
+
+namespace {
+
+constexpr size_t kBlock = 32;  // Matrix.cpp:11
+
+bool insideParallelRegion() {
+#if defined(_OPENMP)
+    return omp_in_parallel() != 0;
+#else
+    return true;
+#endif
+}
+
+// One 32-row band of C += A * B, i-k-j inside 32^3 blocks (Matrix.cpp:24-43).
+void gemmRowBand(const float* a, size_t lda, const float* b, size_t ldb, float* c, size_t ldc,
+                 size_t rowLo, size_t rowHi, size_t n, size_t kTotal) {
+    for (size_t colLo = 0; colLo < n; colLo += kBlock) {
+        const size_t colHi = std::min(colLo + kBlock, n);
+        for (size_t kLo = 0; kLo < kTotal; kLo += kBlock) {
+            const size_t kHi = std::min(kLo + kBlock, kTotal);
+            for (size_t i = rowLo; i < rowHi; ++i) {
+                float* cRow = c + i * ldc;
+                for (size_t kk = kLo; kk < kHi; ++kk) {
+                    const float aik = a[i * lda + kk];
+                    const float* bRow = b + kk * ldb;
+                    for (size_t j = colLo; j < colHi; ++j) cRow[j] += aik * bRow[j];
+                }
+            }
+        }
+    }
+}
+
+// dst (outRows x outCols) = src^T, src is outCols x outRows (Matrix.cpp:14-22)
+void packTranspose(const float* src, size_t srcCols, size_t outRows, size_t outCols, std::vector<float>& dst) {
+    dst.resize(outRows * outCols);
+    for (size_t r = 0; r < outRows; ++r)
+        for (size_t c = 0; c < outCols; ++c) dst[r * outCols + c] = src[c * srcCols + r];
+}
+
+struct Scratch {
+    std::vector<float> packA, packB;
+    std::vector<float> qHead, kHead, vHead, oHead, gHead;  // d x T each
+    std::vector<float> scores, probs, dProbs, dScores;     // T x T each, [key][query]
+    std::vector<float> dqHead, dkHead, dvHead;
+};
+
+// C = op(A) op(B); zero-fill then accumulate (Matrix.cpp:106-148).
+void gemm(const float* a, size_t aRows, size_t aCols, const float* b, size_t bRows, size_t bCols, float* c,
+          bool transA, bool transB, Scratch& scratch) {
+    const size_t m = transA ? aCols : aRows;
+    const size_t kTotal = transA ? aRows : aCols;
+    const size_t n = transB ? bRows : bCols;
+    std::fill(c, c + m * n, 0.0f);
+
+    const float* ap = a;
+    size_t lda = aCols;
+    if (transA) {
+        packTranspose(a, aCols, m, kTotal, scratch.packA);
+        ap = scratch.packA.data();
+        lda = kTotal;
+    }
+    const float* bp = b;
+    size_t ldb = bCols;
+    if (transB) {
+        packTranspose(b, bCols, kTotal, n, scratch.packB);
+        bp = scratch.packB.data();
+        ldb = n;
+    }
+
+    const size_t work = m * kTotal * n;
+    const long bandCount = static_cast<long>((m + kBlock - 1) / kBlock);
+    if (work >= 65536 && !insideParallelRegion()) {  // Matrix.cpp:139-146
+#if defined(_OPENMP)
+#pragma omp parallel for schedule(static)
+#endif
+        for (long band = 0; band < bandCount; ++band) {
+            const size_t lo = static_cast<size_t>(band) * kBlock;
+            gemmRowBand(ap, lda, bp, ldb, c, n, lo, std::min(lo + kBlock, m), n, kTotal);
+        }
+        return;
+    }
+    for (long band = 0; band < bandCount; ++band) {
+        const size_t lo = static_cast<size_t>(band) * kBlock;
+        gemmRowBand(ap, lda, bp, ldb, c, n, lo, std::min(lo + kBlock, m), n, kTotal);
+    }
+}
+
+// Softmax over rows (classes) for every column (Softmax.cpp:10-44).
+void softmaxColumns(const float* logits, float* out, size_t rows, size_t cols) {
+    const bool parallel = cols >= 32 && !insideParallelRegion();
+    (void)parallel;
+#if defined(_OPENMP)
+#pragma omp parallel for schedule(static) if (parallel)
+#endif
+    for (long col = 0; col < static_cast<long>(cols); ++col) {
+        float top = logits[col];
+        for (size_t r = 1; r < rows; ++r)
+            if (logits[r * cols + col] > top) top = logits[r * cols + col];
+        float total = 0.0f;
+        for (size_t r = 0; r < rows; ++r) {
+            const float e = std::exp(logits[r * cols + col] - top);
+            out[r * cols + col] = e;
+            total += e;
+        }
+        for (size_t r = 0; r < rows; ++r) out[r * cols + col] /= total;
+    }
+}
+
+void gatherHead(const float* base, int head, int d, size_t stride, size_t col0, size_t t, std::vector<float>& dst) {
+    dst.resize(static_cast<size_t>(d) * t);
+    for (int r = 0; r < d; ++r)
+        std::memcpy(dst.data() + static_cast<size_t>(r) * t,
+                    base + (static_cast<size_t>(head) * d + r) * stride + col0, t * sizeof(float));
+}
+
+void scatterHead(float* base, int head, int d, size_t stride, size_t col0, size_t t, const float* src, bool add) {
+    for (int r = 0; r < d; ++r) {
+        float* row = base + (static_cast<size_t>(head) * d + r) * stride + col0;
+        const float* s = src + static_cast<size_t>(r) * t;
+        if (add)
+            for (size_t c = 0; c < t; ++c) row[c] += s[c];
+        else
+            std::memcpy(row, s, t * sizeof(float));
+    }
+}
+
+struct Geometry {
+    int qHeads, kvHeads, d;
+    size_t stride, t;
+    float scale;
+    bool causal;
+};
+
+void onePack(const Geometry& g, size_t col0, const float* q, const float* k, const float* v, float* out, float* lse,
+             const float* dOut, float* dq, float* dk, float* dv, Scratch& s) {
+    const size_t t = g.t;
+    const int d = g.d;
+    const int group = g.qHeads / g.kvHeads;  // CausalSelfAttention.cpp:90-93
+    s.scores.resize(t * t);
+    s.probs.resize(t * t);
+    s.oHead.resize(static_cast<size_t>(d) * t);
+
+    if (dOut) {
+        // keyGradient / valueGradient start from zero (CausalSelfAttention.cpp:271-276)
+        for (int h = 0; h < g.kvHeads; ++h)
+            for (int r = 0; r < d; ++r) {
+                const size_t off = (static_cast<size_t>(h) * d + r) * g.stride + col0;
+                std::fill(dk + off, dk + off + t, 0.0f);
+                std::fill(dv + off, dv + off + t, 0.0f);
+            }
+        s.dProbs.resize(t * t);
+        s.dScores.resize(t * t);
+        s.dqHead.resize(static_cast<size_t>(d) * t);
+        s.dkHead.resize(static_cast<size_t>(d) * t);
+        s.dvHead.resize(static_cast<size_t>(d) * t);
+    }
+
+    for (int h = 0; h < g.qHeads; ++h) {
+        const int kvHead = h / group;
+        gatherHead(q, h, d, g.stride, col0, t, s.qHead);
+        gatherHead(k, kvHead, d, g.stride, col0, t, s.kHead);
+        gatherHead(v, kvHead, d, g.stride, col0, t, s.vHead);
+
+        // scores[key][query] = scale * sum_dim K[dim][key] Q[dim][query], then mask (CausalSelfAttention.cpp:122-126)
+        gemm(s.kHead.data(), d, t, s.qHead.data(), d, t, s.scores.data(), true, false, s);
+        for (size_t i = 0; i < t * t; ++i) s.scores[i] *= g.scale;
+        if (g.causal)
+            for (size_t key = 0; key < t; ++key)
+                for (size_t query = 0; query < key && query < t; ++query) s.scores[key * t + query] = -1e9f;
+
+        softmaxColumns(s.scores.data(), s.probs.data(), t, t);
+
+        // attended = V P (CausalSelfAttention.cpp:150-152)
+        gemm(s.vHead.data(), d, t, s.probs.data(), t, t, s.oHead.data(), false, false, s);
+        scatterHead(out, h, d, g.stride, col0, t, s.oHead.data(), false);
+
+        if (lse) {
+            // natural-log LSE of the scaled, masked scores, accumulated in double
+            for (size_t query = 0; query < t; ++query) {
+                float top = s.scores[query];
+                for (size_t key = 1; key < t; ++key) top = std::max(top, s.scores[key * t + query]);
+                double total = 0.0;
+                for (size_t key = 0; key < t; ++key)
+                    total += std::exp(static_cast<double>(s.scores[key * t + query]) - static_cast<double>(top));
+                lse[static_cast<size_t>(h) * g.stride + col0 + query] = static_cast<float>(top + std::log(total));
+            }
+        }
+
+        if (!dOut) continue;
+
+        gatherHead(dOut, h, d, g.stride, col0, t, s.gHead);
+        // dV = dA P^T ; dP = V^T dA (CausalSelfAttention.cpp:334-335)
+        gemm(s.gHead.data(), d, t, s.probs.data(), t, t, s.dvHead.data(), false, true, s);
+        gemm(s.vHead.data(), d, t, s.gHead.data(), d, t, s.dProbs.data(), true, false, s);
+        // softmax jacobian per query column (CausalSelfAttention.cpp:195-210)
+        for (size_t query = 0; query < t; ++query) {
+            float dot = 0.0f;
+            for (size_t key = 0; key < t; ++key) dot += s.dProbs[key * t + query] * s.probs[key * t + query];
+            for (size_t key = 0; key < t; ++key)
+                s.dScores[key * t + query] = s.probs[key * t + query] * (s.dProbs[key * t + query] - dot);
+        }
+        if (g.causal)  // CausalSelfAttention.cpp:338-343
+            for (size_t key = 0; key < t; ++key)
+                for (size_t query = 0; query < key && query < t; ++query) s.dScores[key * t + query] = 0.0f;
+        for (size_t i = 0; i < t * t; ++i) s.dScores[i] *= g.scale;
+        // dQ = K dS ; dK = Q dS^T (CausalSelfAttention.cpp:346-347)
+        gemm(s.kHead.data(), d, t, s.dScores.data(), t, t, s.dqHead.data(), false, false, s);
+        gemm(s.qHead.data(), d, t, s.dScores.data(), t, t, s.dkHead.data(), false, true, s);
+
+        scatterHead(dq, h, d, g.stride, col0, t, s.dqHead.data(), false);
+        scatterHead(dk, kvHead, d, g.stride, col0, t, s.dkHead.data(), true);
+        scatterHead(dv, kvHead, d, g.stride, col0, t, s.dvHead.data(), true);
+    }
+}
+
+}  // namespace
+
+extern "C" int sentinel_oracle_attention(const float* q, const float* k, const float* v, float* out, float* lse,
+                                         const float* d_out, float* dq, float* dk, float* dv, int qHeads, int kvHeads,
+                                         int headDim, int strideColumns, int colStart, int seqLen, int packCount,
+                                         float scale, int causal, int packParallel) {
+    if (!q || !k || !v || !out) return -1;
+    if (qHeads <= 0 || kvHeads <= 0 || headDim <= 0 || qHeads % kvHeads != 0) return -1;
+    if (seqLen <= 0 || packCount <= 0 || colStart < 0) return -1;
+    if (static_cast<long long>(colStart) + static_cast<long long>(packCount) * seqLen > strideColumns) return -1;
+    const bool wantBackward = d_out != nullptr;
+    if (wantBackward != (dq != nullptr) || wantBackward != (dk != nullptr) || wantBackward != (dv != nullptr)) return -1;
+
+    Geometry g{qHeads, kvHeads, headDim, static_cast<size_t>(strideColumns), static_cast<size_t>(seqLen), scale, causal != 0};
+
+    if (packParallel && packCount > 1) {
+#if defined(_OPENMP)
+#pragma omp parallel
+#endif
+        {
+            Scratch scratch;
+#if defined(_OPENMP)
+#pragma omp for schedule(dynamic, 1)
+#endif
+            for (int pack = 0; pack < packCount; ++pack)
+                onePack(g, static_cast<size_t>(colStart) + static_cast<size_t>(pack) * g.t, q, k, v, out, lse, d_out, dq, dk,
+                        dv, scratch);
+        }
+        return 0;
+    }
+    Scratch scratch;
+    for (int pack = 0; pack < packCount; ++pack)
+        onePack(g, static_cast<size_t>(colStart) + static_cast<size_t>(pack) * g.t, q, k, v, out, lse, d_out, dq, dk, dv,
+                scratch);
+    return 0;
+}
+
+extern "C" int sentinel_oracle_delta(const float* out, const float* d_out, float* delta, int qHeads, int headDim,
+                                     int strideColumns, int colStart, int seqLen, int packCount) {
+    if (!out || !d_out || !delta || qHeads <= 0 || headDim <= 0 || seqLen <= 0 || packCount <= 0 || colStart < 0) return -1;
+    if (static_cast<long long>(colStart) + static_cast<long long>(packCount) * seqLen > strideColumns) return -1;
+    const size_t stride = static_cast<size_t>(strideColumns);
+    for (int h = 0; h < qHeads; ++h)
+        for (size_t col = static_cast<size_t>(colStart); col < static_cast<size_t>(colStart) + static_cast<size_t>(packCount) * seqLen; ++col) {
+            float sum = 0.0f;  // CudaFlashAttention.cu:589-594: dims in increasing order, fp32
+            for (int r = 0; r < headDim; ++r) {
+                const size_t idx = (static_cast<size_t>(h) * headDim + r) * stride + col;
+                sum += out[idx] * d_out[idx];
+            }
+            delta[static_cast<size_t>(h) * stride + col] = sum;
+        }
+    return 0;
+}
+
+extern "C" int sentinel_oracle_gemm(const float* a, int aRows, int aCols, const float* b, int bRows, int bCols, float* c,
+                                    int transposeA, int transposeB) {
+    if (!a || !b || !c || aRows <= 0 || aCols <= 0 || bRows <= 0 || bCols <= 0) return -1;
+    const int inner = transposeA ? aRows : aCols;
+    const int innerB = transposeB ? bCols : bRows;
+    if (inner != innerB) return -1;
+    Scratch scratch;
+    gemm(a, aRows, aCols, b, bRows, bCols, c, transposeA != 0, transposeB != 0, scratch);
+    return 0;
+}
+
+extern "C" int sentinel_oracle_softmax_columns(const float* logits, float* out, int rows, int cols) {
+    if (!logits || !out || rows <= 0 || cols <= 0) return -1;
+    softmaxColumns(logits, out, static_cast<size_t>(rows), static_cast<size_t>(cols));
+    return 0;
+}
+
+extern "C" int sentinel_oracle_max_threads(void) {
+#if defined(_OPENMP)
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

@@ -1,0 +1,64 @@
+/*
+ * TEST INFRASTRUCTURE ONLY - CPU oracle for Sentinel's causal attention.
+ *
+ * This is a plain C++ restatement of the host (OpenMP) attention path of
+ * ToldByNun/sentinel, used to check the HIP kernels and as the CPU baseline
+ * in bench.py.  Nothing in the shipped library links, loads or calls it.
+ *
+ * Tensors use Sentinel's device layout (Cuda/CudaFlashAttention.cu:129-135):
+ *   element(head, dim, column) = base[(head * headDim + dim) * strideColumns + column]
+ * with packCount sequences of seqLen columns starting at colStart.  q / d_out /
+ * out / dq have qHeads heads, k / v / dk / dv have kvHeads heads, lse is
+ * qHeads x strideColumns.
+ */
+#ifndef SENTINEL_ATTENTION_ORACLE_H
+#define SENTINEL_ATTENTION_ORACLE_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Forward (and backward when d_out != NULL) of causal multi-head attention.
+ *
+ *  out, lse            forward results (lse may be NULL); columns outside the
+ *                      pack window are left untouched
+ *  d_out, dq, dk, dv   backward: all four non-NULL or all four NULL; dk / dv
+ *                      are OVERWRITTEN inside the pack window (zero, then the
+ *                      group's query heads are added in increasing order)
+ *  causal              1 = Sentinel's mask (key > query forbidden); 0 = no mask
+ *                      (the CPU reference has no such mode; kept for the device
+ *                      API's `causal` flag)
+ *  packParallel        1 = OpenMP over packs with serial inner loops (mirrors
+ *                      the train loop, Network/LanguageModel.cpp:1109-1125);
+ *                      0 = packs in order, gemm / softmax internally parallel
+ *                      under the reference's own thresholds
+ *
+ * Returns 0, or -1 on invalid geometry.
+ */
+int sentinel_oracle_attention(const float* q, const float* k, const float* v,
+                              float* out, float* lse,
+                              const float* d_out, float* dq, float* dk, float* dv,
+                              int qHeads, int kvHeads, int headDim,
+                              int strideColumns, int colStart, int seqLen, int packCount,
+                              float scale, int causal, int packParallel);
+
+/* D[head][column] = sum_dim out * d_out (Cuda/CudaFlashAttention.cu:576-596). */
+int sentinel_oracle_delta(const float* out, const float* d_out, float* delta,
+                          int qHeads, int headDim, int strideColumns, int colStart,
+                          int seqLen, int packCount);
+
+/* C = op(A) * op(B) with the reference's blocking and summation order
+ * (Math/Matrix.cpp:106-148); exported so tests can pin it on its own. */
+int sentinel_oracle_gemm(const float* a, int aRows, int aCols, const float* b, int bRows, int bCols,
+                         float* c, int transposeA, int transposeB);
+
+/* column softmax (Activations/Softmax.cpp:10-44); rows x cols, row-major */
+int sentinel_oracle_softmax_columns(const float* logits, float* out, int rows, int cols);
+
+int sentinel_oracle_max_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,74 @@
+"""Writes the golden fixtures in this directory from the reference's own compiled CPU attention.
+
+Run in a container that has the reference checkout:  make -C oracle ref && python tests/golden/make_fixtures.py
+Every fixture stores its inputs and the outputs of oracle/_ref (the reference's Matrix / Softmax /
+CausalSelfAttention sources compiled in place), so the tests need neither the reference nor this script.
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+import oracle_lib  # noqa: E402
+
+# name: (q_heads, kv_heads, head_dim, seq_len, packs, col_start, pad_cols, seed, sigma_qk)
+CASES = {
+    "c1_tiny_fp32": (4, 4, 16, 48, 4, 0, 0, 0x5E17 + 1, 1.0),       # the quickstart LM attention shape
+    "gqa_8q2kv_d8_T16": (8, 2, 8, 16, 1, 0, 0, 0x5E17 + 11, 1.0),    # shape of the reference's GQA host smoke
+    "d64_T132": (2, 2, 64, 132, 1, 0, 0, 0x5E17 + 12, 1.0),          # ragged tail past two 64-wide tiles
+    "gqa_d128_T96_B2": (2, 1, 128, 96, 2, 0, 0, 0x5E17 + 13, 1.0),   # head_dim 128, grouped K/V, two packs
+    "d64_T256_B2_window": (1, 1, 64, 256, 2, 8, 24, 0x5E17 + 14, 1.0),  # pack window inside a wider matrix
+    "d32_T80_sharp": (2, 2, 32, 80, 1, 0, 0, 0x5E17 + 15, 3.0),      # sigma 3 queries / keys: peaked softmax
+}
+
+
+def lcg_uniform(count, state):
+    """The reference's smoke-test input recipe (Layers/CausalSelfAttention.cpp:566-574)."""
+    out = np.empty(count, dtype=np.float32)
+    for i in range(count):
+        state = (state * 1664525 + 1013904223) & 0xFFFFFFFF
+        out[i] = np.float32(np.float32(state >> 8) / np.float32(16777216.0)) * np.float32(2.0) - np.float32(1.0)
+    return out, state
+
+
+def main():
+    ref = oracle_lib.reference()
+    if ref is None:
+        raise SystemExit("oracle/_ref is not built (needs the reference checkout): make -C oracle ref")
+    for name, (hq, hkv, d, t, packs, col0, pad, seed, sigma) in CASES.items():
+        rng = np.random.default_rng(seed)
+        stride = col0 + packs * t + pad
+        q = (sigma * rng.standard_normal((hq * d, stride))).astype(np.float32)
+        k = (sigma * rng.standard_normal((hkv * d, stride))).astype(np.float32)
+        v = rng.standard_normal((hkv * d, stride)).astype(np.float32)
+        g = rng.standard_normal((hq * d, stride)).astype(np.float32)
+        res = oracle_lib.oracle_attention(q, k, v, g, q_heads=hq, kv_heads=hkv, head_dim=d, seq_len=t, pack_count=packs,
+                                          col_start=col0, lib="ref")
+        np.savez_compressed(os.path.join(HERE, name + ".npz"), q=q, k=k, v=v, d_out=g,
+                            geometry=np.array([hq, hkv, d, t, packs, col0, stride], dtype=np.int64), **res)
+        print(name, {key: val.shape for key, val in res.items()})
+
+    # gemm / softmax known answers from the reference's Matrix::gemm and Softmax::applyInto
+    rng = np.random.default_rng(0x5E17 + 20)
+    kat = {}
+    for tag, (m, kk, n, ta, tb) in {"nn_33x70x45": (33, 70, 45, False, False), "tn_96x16x96": (96, 16, 96, True, False),
+                                    "nt_16x100x40": (16, 100, 40, False, True), "tt_37x41x29": (37, 41, 29, True, True)}.items():
+        a = rng.standard_normal((kk, m) if ta else (m, kk)).astype(np.float32)
+        b = rng.standard_normal((n, kk) if tb else (kk, n)).astype(np.float32)
+        kat[f"gemm_{tag}_a"], kat[f"gemm_{tag}_b"] = a, b
+        kat[f"gemm_{tag}_c"] = oracle_lib.gemm(a, b, ta, tb, lib="ref")
+        kat[f"gemm_{tag}_flags"] = np.array([ta, tb], dtype=np.int64)
+    logits = (4.0 * rng.standard_normal((50, 37))).astype(np.float32)
+    logits[10:, 3] = -1e9
+    kat["softmax_in"] = logits
+    kat["softmax_out"] = oracle_lib.softmax_columns(logits, lib="ref")
+    lcg, _ = lcg_uniform(64 * 16, 123)
+    kat["lcg_seed123_first1024"] = lcg
+    np.savez_compressed(os.path.join(HERE, "gemm_softmax_kat.npz"), **kat)
+    print("gemm_softmax_kat", len(kat), "arrays")
+
+
+if __name__ == "__main__":
+    main()

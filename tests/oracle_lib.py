@@ -1,0 +1,129 @@
+"""ctypes access to the CPU oracle (oracle/) and, where built, the compiled reference (oracle/_ref).
+
+Test infrastructure only: the shipped package never imports this module.
+All tensors are float32 numpy arrays in Sentinel's device layout,
+``[(head * head_dim + dim), column]`` with ``stride`` columns per row.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_SO = os.path.join(ORACLE_DIR, "libsentinel_attention_oracle.so")
+REF_SO = os.path.join(ORACLE_DIR, "_ref", "libsentinel_ref_attention.so")
+
+_fp = ctypes.POINTER(ctypes.c_float)
+
+
+def _ptr(a):
+    if a is None:
+        return None
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_fp)
+
+
+def build_oracle(force=False):
+    """Compile the oracle with the committed Makefile when it is missing (CPU only, about 3 s)."""
+    if force or not os.path.exists(ORACLE_SO):
+        subprocess.run(["make", "-C", ORACLE_DIR, "oracle"], check=True, capture_output=True)
+    return ORACLE_SO
+
+
+_oracle = None
+_ref = None
+
+
+def oracle():
+    global _oracle
+    if _oracle is None:
+        lib = ctypes.CDLL(build_oracle())
+        lib.sentinel_oracle_attention.argtypes = [_fp] * 9 + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int, ctypes.c_int]
+        lib.sentinel_oracle_attention.restype = ctypes.c_int
+        lib.sentinel_oracle_delta.argtypes = [_fp] * 3 + [ctypes.c_int] * 6
+        lib.sentinel_oracle_gemm.argtypes = [_fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int]
+        lib.sentinel_oracle_softmax_columns.argtypes = [_fp, _fp, ctypes.c_int, ctypes.c_int]
+        lib.sentinel_oracle_max_threads.restype = ctypes.c_int
+        _oracle = lib
+    return _oracle
+
+
+def reference():
+    """The reference's own compiled CPU path, or None when oracle/_ref was not built."""
+    global _ref
+    if _ref is None:
+        if not os.path.exists(REF_SO):
+            return None
+        lib = ctypes.CDLL(REF_SO)
+        lib.sentinel_ref_attention.argtypes = [_fp] * 9 + [ctypes.c_int] * 8
+        lib.sentinel_ref_gemm.argtypes = [_fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int]
+        lib.sentinel_ref_softmax_columns.argtypes = [_fp, _fp, ctypes.c_int, ctypes.c_int]
+        _ref = lib
+    return _ref
+
+
+def _alloc_like(x, fill=np.nan):
+    return np.full_like(x, fill)
+
+
+def oracle_attention(q, k, v, d_out=None, *, q_heads, kv_heads, head_dim, seq_len, pack_count=1, col_start=0,
+                     scale=None, causal=True, pack_parallel=False, lib="oracle", per_head=False):
+    """Run forward (+ backward when d_out is given). Returns dict(out, lse[, dq, dk, dv]).
+
+    Untouched columns (outside the pack window) come back as NaN so tests can check they were left alone.
+    """
+    stride = q.shape[1]
+    assert q.shape[0] == q_heads * head_dim and k.shape == v.shape == (kv_heads * head_dim, stride)
+    if scale is None:
+        scale = np.float32(1.0) / np.sqrt(np.float32(head_dim))
+    out = _alloc_like(q)
+    lse = np.full((q_heads, stride), np.nan, dtype=np.float32)
+    dq = dk = dv = None
+    if d_out is not None:
+        dq, dk, dv = _alloc_like(q), _alloc_like(k), _alloc_like(v)
+    if lib == "oracle":
+        rc = oracle().sentinel_oracle_attention(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out), _ptr(dq),
+                                                 _ptr(dk), _ptr(dv), q_heads, kv_heads, head_dim, stride, col_start,
+                                                 seq_len, pack_count, float(scale), int(causal), int(pack_parallel))
+    else:
+        assert causal and abs(float(scale) - 1.0 / np.sqrt(head_dim)) < 1e-7
+        rc = reference().sentinel_ref_attention(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out), _ptr(dq),
+                                                 _ptr(dk), _ptr(dv), q_heads, kv_heads, head_dim, stride, col_start,
+                                                 seq_len, pack_count, int(per_head))
+    if rc != 0:
+        raise ValueError(f"{lib} attention returned {rc}")
+    res = {"out": out, "lse": lse}
+    if d_out is not None:
+        res.update(dq=dq, dk=dk, dv=dv)
+    return res
+
+
+def oracle_delta(out, d_out, *, q_heads, head_dim, seq_len, pack_count=1, col_start=0):
+    stride = out.shape[1]
+    delta = np.full((q_heads, stride), np.nan, dtype=np.float32)
+    rc = oracle().sentinel_oracle_delta(_ptr(out), _ptr(d_out), _ptr(delta), q_heads, head_dim, stride, col_start, seq_len, pack_count)
+    if rc != 0:
+        raise ValueError(f"oracle delta returned {rc}")
+    return delta
+
+
+def gemm(a, b, trans_a=False, trans_b=False, lib="oracle"):
+    m = a.shape[1] if trans_a else a.shape[0]
+    n = b.shape[0] if trans_b else b.shape[1]
+    c = np.empty((m, n), dtype=np.float32)
+    fn = oracle().sentinel_oracle_gemm if lib == "oracle" else reference().sentinel_ref_gemm
+    rc = fn(_ptr(a), a.shape[0], a.shape[1], _ptr(b), b.shape[0], b.shape[1], _ptr(c), int(trans_a), int(trans_b))
+    if rc != 0:
+        raise ValueError(f"{lib} gemm returned {rc}")
+    return c
+
+
+def softmax_columns(x, lib="oracle"):
+    y = np.empty_like(x)
+    fn = oracle().sentinel_oracle_softmax_columns if lib == "oracle" else reference().sentinel_ref_softmax_columns
+    rc = fn(_ptr(x), _ptr(y), x.shape[0], x.shape[1])
+    if rc != 0:
+        raise ValueError(f"{lib} softmax returned {rc}")
+    return y
