@@ -1,0 +1,118 @@
+/*
+ * sentinel_hip_attn.h - C ABI of the MI355X (gfx950) causal flash-attention forward / backward.
+ *
+ * These entry points stand where Sentinel's CUDA attention dispatch stands: they take the same
+ * tensors, geometry and column window as
+ *     CudaFlashAttention::forwardMultiHead   (sentinel/NeuralNet/Cuda/CudaFlashAttention.hpp:30,
+ *                                             sentinel/NeuralNet/Cuda/CudaFlashAttention.cu:1543-1609)
+ *     CudaFlashAttention::backwardMultiHead  (sentinel/NeuralNet/Cuda/CudaFlashAttention.hpp:40,
+ *                                             sentinel/NeuralNet/Cuda/CudaFlashAttention.cu:1615-1700)
+ * as called from CudaCausalSelfAttention::attendFullSequence / ::backward
+ * (sentinel/NeuralNet/Cuda/CudaCausalSelfAttention.cu:237-249, :421-438), but as plain pointers and
+ * sizes: the caller owns every buffer, nothing is allocated, freed or synchronised inside a call, and
+ * all work is enqueued on the stream that is passed in (capture-safe).
+ *
+ * Differences from the CUDA path they replace, all additive:
+ *   - head_dim up to 128 (the CUDA path stops at 64, CudaFlashAttention.hpp:16);
+ *   - grouped-query attention is native: k / v / dk / dv have kv_heads heads and query head h reads
+ *     kv head h / (q_heads / kv_heads), so no expanded K/V copies and no gradient reduction pass
+ *     (replaces expandKvHeadsInto / reduceKvHeadGradsInto, CudaCausalSelfAttention.cu:27-44);
+ *   - dq, dk and dv are overwritten deterministically (no atomics); pre-zeroed buffers, as the
+ *     CUDA caller provides (CudaCausalSelfAttention.cu:392-394), are fine but not required;
+ *   - any seq_len >= 1 and any stride are accepted (no multiple-of-4 rule).
+ */
+#ifndef SENTINEL_HIP_ATTN_H
+#define SENTINEL_HIP_ATTN_H
+
+#include <stddef.h>
+
+#if defined(__GNUC__)
+#define SENTINEL_HIP_API __attribute__((visibility("default")))
+#else
+#define SENTINEL_HIP_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Return codes. The C++ shim maps INVALID_ARGUMENT and UNSUPPORTED to std::invalid_argument and
+ * RUNTIME to std::runtime_error, the exception types of validateMultiHeadShape / resolveColumnWindow
+ * (CudaFlashAttention.cu:1458-1471, :1533-1539) and throwIfCudaFailed (:1608). */
+enum {
+    SENTINEL_HIP_OK = 0,
+    SENTINEL_HIP_INVALID_ARGUMENT = 1, /* null pointer, bad head geometry, bad column window */
+    SENTINEL_HIP_UNSUPPORTED = 2,      /* head_dim / dtype / layout combination has no kernel: use the dense path */
+    SENTINEL_HIP_RUNTIME = 3           /* no device, launch failure */
+};
+
+/* element type of q, k, v, out, d_out, dq, dk, dv (lse and delta are always float) */
+enum { SENTINEL_HIP_F32 = 0, SENTINEL_HIP_BF16 = 1, SENTINEL_HIP_F16 = 2 };
+
+/* arithmetic used for the matrix products */
+enum {
+    SENTINEL_HIP_COMPUTE_AUTO = -1, /* F32 io -> F32 arithmetic; BF16 / F16 io -> MFMA in that type */
+    SENTINEL_HIP_COMPUTE_F32 = 0,   /* exact fp32 FMA path (any head_dim <= 128) */
+    SENTINEL_HIP_COMPUTE_BF16 = 1,  /* bf16 MFMA, fp32 accumulation (head_dim 64 or 128) */
+    SENTINEL_HIP_COMPUTE_F16 = 2    /* fp16 MFMA, fp32 accumulation (head_dim 64 or 128) */
+};
+
+/*
+ * Tensor layouts.
+ *  SENTINEL_HIP_LAYOUT_COLUMNS  Sentinel's device layout (CudaFlashAttention.cu:129-135):
+ *        element(head, dim, column) = base[(head * head_dim + dim) * stride_columns + column]
+ *        pack p occupies columns [column_start + p * seq_len, column_start + (p + 1) * seq_len);
+ *        lse is q_heads x stride_columns. Columns outside the pack window are never written.
+ *  SENTINEL_HIP_LAYOUT_BHTD     contiguous [pack_count, heads, seq_len, head_dim]; lse is
+ *        [pack_count, q_heads, seq_len]; stride_columns and column_start are ignored.
+ * delta workspace (both layouts): q_heads x (pack_count * seq_len) floats, the shape the CUDA caller
+ * keeps in CudaCausalSelfAttention::flashDelta (CudaFlashAttention.cu:1640).
+ */
+enum { SENTINEL_HIP_LAYOUT_COLUMNS = 0, SENTINEL_HIP_LAYOUT_BHTD = 1 };
+
+/*
+ * Scratch the caller must provide for a configuration (bytes; 0 when none is needed). Only the
+ * COLUMNS layout with MFMA arithmetic needs any (type-converted [B,H,T,d] copies of the operands).
+ * `backward` != 0 sizes it for sentinel_hip_flash_bwd, else for sentinel_hip_flash_fwd.
+ */
+SENTINEL_HIP_API size_t sentinel_hip_flash_workspace_bytes(int io_dtype, int compute_dtype, int layout, int q_heads, int kv_heads,
+                                          int head_dim, int seq_len, int pack_count, int backward);
+
+/*
+ * out = softmax(scale * Q K^T [+ causal mask]) V and lse = max + ln(sum exp) per query, natural log of
+ * the scaled scores (CudaFlashAttention.cu:1260-1264). Replaces CudaFlashAttention::forwardMultiHead.
+ * `scale` must be positive and finite (the caller passes 1/sqrt(head_dim), CudaCausalSelfAttention.cu:212).
+ * `stream` is a hipStream_t (NULL = default stream).
+ */
+SENTINEL_HIP_API int sentinel_hip_flash_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int io_dtype,
+                           int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim, int stride_columns,
+                           int column_start, int seq_len, int pack_count, float scale, int causal, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/*
+ * dq, dk, dv from d_out with P recomputed from lse and D = rowsum(d_out * out) written to `delta`.
+ * Replaces CudaFlashAttention::backwardMultiHead (which launches the Delta kernel and one backward
+ * kernel, CudaFlashAttention.cu:1640-1699).
+ */
+SENTINEL_HIP_API int sentinel_hip_flash_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                           const void* d_out, void* dq, void* dk, void* dv, float* delta, int io_dtype,
+                           int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim, int stride_columns,
+                           int column_start, int seq_len, int pack_count, float scale, int causal, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/* Largest head_dim any kernel here accepts (the CUDA path's CudaFlashAttention::maxHeadDimension is 64). */
+SENTINEL_HIP_API int sentinel_hip_flash_max_head_dim(void);
+
+/* 1 when a HIP device is usable (stands for CudaMatmul::isAvailable, CudaFlashAttention.cu:1545). */
+SENTINEL_HIP_API int sentinel_hip_device_available(void);
+
+/* Fixed text for a return code. */
+SENTINEL_HIP_API const char* sentinel_hip_strerror(int code);
+
+/* Detail of the last non-OK return on the calling thread ("" if none). */
+SENTINEL_HIP_API const char* sentinel_hip_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SENTINEL_HIP_ATTN_H */

@@ -1,0 +1,8 @@
+"""MI355X-native causal flash attention behind Sentinel's CudaFlashAttention interface."""
+from .flash_attention import (  # noqa: F401
+    HipFlashAttention,
+    flash_attention_backward,
+    flash_attention_forward,
+    library_path,
+    load_library,
+)

@@ -1,0 +1,309 @@
+// C ABI of the attention library: argument validation, layout resolution and kernel dispatch.
+// Validation follows CudaFlashAttention's host code (sentinel/NeuralNet/Cuda/CudaFlashAttention.cu:
+// validateMultiHeadShape :1458-1471, resolveColumnWindow :1533-1539, pack window :1551-1552,
+// device check :1545-1546) with return codes in place of exceptions.
+#include "../../include/sentinel_hip_attn.h"
+
+#include "flash_common.h"
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+using namespace sentinel_hip;
+
+namespace {
+
+thread_local char g_last_error[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list args;
+    va_start(args, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, args);
+    va_end(args);
+    return code;
+}
+
+int fail_hip(const char* what, hipError_t err) {
+    return fail(SENTINEL_HIP_RUNTIME, "%s: %s", what, hipGetErrorString(err));
+}
+
+size_t align_up(size_t x) { return (x + 255) & ~static_cast<size_t>(255); }
+
+struct Resolved {
+    AttnGeom g;
+    int io;        // SENTINEL_HIP_F32 / BF16 / F16
+    int compute;   // resolved compute type
+    int layout;
+    long long stride;  // column layout only
+    int column_start;
+    bool adapter;  // column layout fp32 tensors converted to [B,H,T,d] 16-bit for the MFMA kernels
+};
+
+// Geometry checks shared by both entry points. `op` names the operation in messages.
+int resolve(const char* op, int io_dtype, int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+            int stride_columns, int column_start, int seq_len, int pack_count, float scale, int causal, Resolved* r) {
+    if (io_dtype < SENTINEL_HIP_F32 || io_dtype > SENTINEL_HIP_F16) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s unknown io dtype %d", op, io_dtype);
+    if (compute_dtype < SENTINEL_HIP_COMPUTE_AUTO || compute_dtype > SENTINEL_HIP_COMPUTE_F16)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s unknown compute dtype %d", op, compute_dtype);
+    if (layout != SENTINEL_HIP_LAYOUT_COLUMNS && layout != SENTINEL_HIP_LAYOUT_BHTD)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s unknown layout %d", op, layout);
+    if (q_heads <= 0 || head_dim <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s invalid head geometry", op);
+    if (kv_heads <= 0) kv_heads = q_heads;
+    if (q_heads % kv_heads != 0)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s headCount must be divisible by kvHeadCount", op);
+    if (head_dim > sentinel_hip_flash_max_head_dim())
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s headDim exceeds maxHeadDimension", op);
+    if (pack_count <= 0) pack_count = 1;
+    if (layout == SENTINEL_HIP_LAYOUT_COLUMNS) {
+        if (stride_columns <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
+        if (seq_len <= 0) seq_len = stride_columns - column_start;  // resolveColumnWindow
+        if (column_start < 0 || seq_len <= 0 || (long long)column_start + seq_len > stride_columns)
+            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s invalid column window", op);
+        if ((long long)column_start + (long long)pack_count * seq_len > stride_columns)
+            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s pack window exceeds columns", op);
+    } else {
+        if (seq_len <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
+        stride_columns = 0;
+        column_start = 0;
+    }
+    if (!(scale > 0.0f) || !std::isfinite(scale))
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s scale must be positive and finite", op);
+
+    int compute = compute_dtype;
+    if (compute == SENTINEL_HIP_COMPUTE_AUTO) compute = io_dtype;
+    bool adapter = false;
+    if (compute == SENTINEL_HIP_COMPUTE_F32) {
+        if (io_dtype != SENTINEL_HIP_F32)
+            return fail(SENTINEL_HIP_UNSUPPORTED, "%s fp32 arithmetic needs fp32 tensors", op);
+    } else {
+        if (!mfma_supported(head_dim))
+            return fail(SENTINEL_HIP_UNSUPPORTED, "%s MFMA kernels cover head_dim 64 and 128, got %d", op, head_dim);
+        if (io_dtype == SENTINEL_HIP_F32) {
+            if (layout != SENTINEL_HIP_LAYOUT_COLUMNS)
+                return fail(SENTINEL_HIP_UNSUPPORTED, "%s fp32 tensors with MFMA arithmetic need the column layout", op);
+            adapter = true;
+        } else {
+            if (io_dtype != compute)
+                return fail(SENTINEL_HIP_UNSUPPORTED, "%s 16-bit tensors must be multiplied in their own type", op);
+            if (layout != SENTINEL_HIP_LAYOUT_BHTD)
+                return fail(SENTINEL_HIP_UNSUPPORTED, "%s 16-bit tensors need the [B,H,T,d] layout", op);
+        }
+    }
+    // every kernel indexes one tensor with 64-bit offsets but tiles with int
+    if ((long long)pack_count * seq_len > 0x7fffffffLL / 4)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s too many columns", op);
+
+    r->g = AttnGeom{q_heads, kv_heads, head_dim, seq_len, pack_count, scale, causal ? 1 : 0};
+    r->io = io_dtype;
+    r->compute = compute;
+    r->layout = layout;
+    r->stride = stride_columns;
+    r->column_start = column_start;
+    r->adapter = adapter;
+    return SENTINEL_HIP_OK;
+}
+
+TensorMap tensor_map(const Resolved& r, int heads) {
+    if (r.layout == SENTINEL_HIP_LAYOUT_COLUMNS)
+        return TensorMap{r.g.seq_len, (long long)r.g.head_dim * r.stride, 1, r.stride};
+    return TensorMap{(long long)heads * r.g.seq_len * r.g.head_dim, (long long)r.g.seq_len * r.g.head_dim, r.g.head_dim, 1};
+}
+
+RowMap lse_map(const Resolved& r) {
+    if (r.layout == SENTINEL_HIP_LAYOUT_COLUMNS) return RowMap{r.g.seq_len, r.stride};
+    return RowMap{(long long)r.g.q_heads * r.g.seq_len, r.g.seq_len};
+}
+
+bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+size_t q_bytes16(const AttnGeom& g) { return align_up((size_t)g.packs * g.q_heads * g.seq_len * g.head_dim * 2); }
+size_t kv_bytes16(const AttnGeom& g) { return align_up((size_t)g.packs * g.kv_heads * g.seq_len * g.head_dim * 2); }
+
+size_t workspace_need(const Resolved& r, bool backward) {
+    if (!r.adapter) return 0;
+    const size_t nq = q_bytes16(r.g);
+    const size_t nkv = kv_bytes16(r.g);
+    return backward ? 4 * nq + 4 * nkv : 2 * nq + 2 * nkv;
+}
+
+}  // namespace
+
+extern "C" int sentinel_hip_flash_max_head_dim(void) { return 128; }
+
+extern "C" int sentinel_hip_device_available(void) {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return count > 0 ? 1 : 0;
+}
+
+extern "C" const char* sentinel_hip_strerror(int code) {
+    switch (code) {
+        case SENTINEL_HIP_OK: return "ok";
+        case SENTINEL_HIP_INVALID_ARGUMENT: return "invalid argument";
+        case SENTINEL_HIP_UNSUPPORTED: return "unsupported configuration";
+        case SENTINEL_HIP_RUNTIME: return "HIP runtime failure";
+        default: return "unknown code";
+    }
+}
+
+extern "C" const char* sentinel_hip_last_error(void) { return g_last_error; }
+
+extern "C" size_t sentinel_hip_flash_workspace_bytes(int io_dtype, int compute_dtype, int layout, int q_heads, int kv_heads,
+                                                     int head_dim, int seq_len, int pack_count, int backward) {
+    Resolved r;
+    // stride / window are irrelevant to the size: use a window that always validates
+    const int packs = pack_count <= 0 ? 1 : pack_count;
+    if (seq_len <= 0) return 0;
+    if ((long long)packs * seq_len > 0x7fffffffLL / 4) return 0;
+    if (resolve("sentinel_hip_flash_workspace_bytes", io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim,
+                packs * seq_len, 0, seq_len, packs, 1.0f, 1, &r) != SENTINEL_HIP_OK)
+        return 0;
+    return workspace_need(r, backward != 0);
+}
+
+extern "C" int sentinel_hip_flash_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int io_dtype,
+                                      int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+                                      int stride_columns, int column_start, int seq_len, int pack_count, float scale,
+                                      int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
+    const char* op = "sentinel_hip_flash_fwd";
+    if (!q || !k || !v || !out || !lse) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
+    Resolved r;
+    const int rc = resolve(op, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns, column_start,
+                           seq_len, pack_count, scale, causal, &r);
+    if (rc != SENTINEL_HIP_OK) return rc;
+    if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
+    hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
+    const AttnGeom& g = r.g;
+
+    if (r.compute == SENTINEL_HIP_COMPUTE_F32) {
+        const long long off = r.column_start;
+        const hipError_t err = launch_fwd_f32(static_cast<const float*>(q) + off, static_cast<const float*>(k) + off,
+                                              static_cast<const float*>(v) + off, static_cast<float*>(out) + off, lse + off,
+                                              tensor_map(r, g.q_heads), tensor_map(r, g.kv_heads), lse_map(r), g, stream);
+        if (err != hipSuccess) return fail_hip("fp32 forward launch", err);
+        return SENTINEL_HIP_OK;
+    }
+
+    const Elem type = static_cast<Elem>(r.compute);
+    if (!r.adapter) {
+        if (misaligned(q) || misaligned(k) || misaligned(v) || misaligned(out))
+            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s 16-bit tensors must be 16-byte aligned", op);
+        const hipError_t err = launch_fwd_mfma(type, q, k, v, out, lse, lse_map(r), g, stream);
+        if (err != hipSuccess) return fail_hip("MFMA forward launch", err);
+        return SENTINEL_HIP_OK;
+    }
+
+    // column-layout fp32 tensors: convert operands, run the MFMA kernel, convert the result back
+    const size_t need = workspace_need(r, false);
+    if (!workspace || workspace_bytes < need || misaligned(workspace))
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s needs %zu bytes of 16-byte aligned workspace", op, need);
+    char* ws = static_cast<char*>(workspace);
+    void* q16 = ws;
+    void* o16 = ws + q_bytes16(g);
+    void* k16 = ws + 2 * q_bytes16(g);
+    void* v16 = ws + 2 * q_bytes16(g) + kv_bytes16(g);
+    const long long off = r.column_start;
+    const int stride = static_cast<int>(r.stride);
+    hipError_t err = launch_columns_to_bhtd(type, static_cast<const float*>(q) + off, q16, g.q_heads, g.head_dim, stride,
+                                            g.seq_len, g.packs, stream);
+    if (err == hipSuccess)
+        err = launch_columns_to_bhtd(type, static_cast<const float*>(k) + off, k16, g.kv_heads, g.head_dim, stride,
+                                     g.seq_len, g.packs, stream);
+    if (err == hipSuccess)
+        err = launch_columns_to_bhtd(type, static_cast<const float*>(v) + off, v16, g.kv_heads, g.head_dim, stride,
+                                     g.seq_len, g.packs, stream);
+    if (err == hipSuccess) err = launch_fwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g, stream);
+    if (err == hipSuccess)
+        err = launch_bhtd_to_columns(type, o16, static_cast<float*>(out) + off, g.q_heads, g.head_dim, stride, g.seq_len,
+                                     g.packs, stream);
+    if (err != hipSuccess) return fail_hip("MFMA forward (column layout) launch", err);
+    return SENTINEL_HIP_OK;
+}
+
+extern "C" int sentinel_hip_flash_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                                      const void* d_out, void* dq, void* dk, void* dv, float* delta, int io_dtype,
+                                      int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+                                      int stride_columns, int column_start, int seq_len, int pack_count, float scale,
+                                      int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
+    const char* op = "sentinel_hip_flash_bwd";
+    if (!q || !k || !v || !out || !lse || !d_out || !dq || !dk || !dv || !delta)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
+    Resolved r;
+    const int rc = resolve(op, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns, column_start,
+                           seq_len, pack_count, scale, causal, &r);
+    if (rc != SENTINEL_HIP_OK) return rc;
+    if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
+    hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
+    const AttnGeom& g = r.g;
+
+    if (r.compute == SENTINEL_HIP_COMPUTE_F32) {
+        const long long off = r.column_start;
+        const hipError_t err = launch_bwd_f32(
+            static_cast<const float*>(q) + off, static_cast<const float*>(k) + off, static_cast<const float*>(v) + off,
+            static_cast<const float*>(out) + off, lse + off, static_cast<const float*>(d_out) + off,
+            static_cast<float*>(dq) + off, static_cast<float*>(dk) + off, static_cast<float*>(dv) + off, delta,
+            tensor_map(r, g.q_heads), tensor_map(r, g.kv_heads), lse_map(r), g, stream);
+        if (err != hipSuccess) return fail_hip("fp32 backward launch", err);
+        return SENTINEL_HIP_OK;
+    }
+
+    const Elem type = static_cast<Elem>(r.compute);
+    if (!r.adapter) {
+        if (misaligned(q) || misaligned(k) || misaligned(v) || misaligned(out) || misaligned(d_out) || misaligned(dq) ||
+            misaligned(dk) || misaligned(dv))
+            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s 16-bit tensors must be 16-byte aligned", op);
+        const hipError_t err = launch_bwd_mfma(type, q, k, v, out, lse, lse_map(r), d_out, dq, dk, dv, delta, g, stream);
+        if (err != hipSuccess) return fail_hip("MFMA backward launch", err);
+        return SENTINEL_HIP_OK;
+    }
+
+    const size_t need = workspace_need(r, true);
+    if (!workspace || workspace_bytes < need || misaligned(workspace))
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s needs %zu bytes of 16-byte aligned workspace", op, need);
+    char* ws = static_cast<char*>(workspace);
+    const size_t nq = q_bytes16(g);
+    const size_t nkv = kv_bytes16(g);
+    void* q16 = ws;
+    void* o16 = ws + nq;
+    void* g16 = ws + 2 * nq;
+    void* dq16 = ws + 3 * nq;
+    void* k16 = ws + 4 * nq;
+    void* v16 = ws + 4 * nq + nkv;
+    void* dk16 = ws + 4 * nq + 2 * nkv;
+    void* dv16 = ws + 4 * nq + 3 * nkv;
+    const long long off = r.column_start;
+    const int stride = static_cast<int>(r.stride);
+    const int T = g.seq_len;
+    hipError_t err = launch_columns_to_bhtd(type, static_cast<const float*>(q) + off, q16, g.q_heads, g.head_dim, stride, T,
+                                            g.packs, stream);
+    if (err == hipSuccess)
+        err = launch_columns_to_bhtd(type, static_cast<const float*>(out) + off, o16, g.q_heads, g.head_dim, stride, T,
+                                     g.packs, stream);
+    if (err == hipSuccess)
+        err = launch_columns_to_bhtd(type, static_cast<const float*>(d_out) + off, g16, g.q_heads, g.head_dim, stride, T,
+                                     g.packs, stream);
+    if (err == hipSuccess)
+        err = launch_columns_to_bhtd(type, static_cast<const float*>(k) + off, k16, g.kv_heads, g.head_dim, stride, T,
+                                     g.packs, stream);
+    if (err == hipSuccess)
+        err = launch_columns_to_bhtd(type, static_cast<const float*>(v) + off, v16, g.kv_heads, g.head_dim, stride, T,
+                                     g.packs, stream);
+    if (err == hipSuccess)
+        err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream);
+    if (err == hipSuccess)
+        err = launch_bhtd_to_columns(type, dq16, static_cast<float*>(dq) + off, g.q_heads, g.head_dim, stride, T, g.packs,
+                                     stream);
+    if (err == hipSuccess)
+        err = launch_bhtd_to_columns(type, dk16, static_cast<float*>(dk) + off, g.kv_heads, g.head_dim, stride, T, g.packs,
+                                     stream);
+    if (err == hipSuccess)
+        err = launch_bhtd_to_columns(type, dv16, static_cast<float*>(dv) + off, g.kv_heads, g.head_dim, stride, T, g.packs,
+                                     stream);
+    if (err != hipSuccess) return fail_hip("MFMA backward (column layout) launch", err);
+    return SENTINEL_HIP_OK;
+}

@@ -1,0 +1,65 @@
+// Internal declarations shared by the attention kernels and the C ABI (not installed).
+#ifndef SENTINEL_HIP_FLASH_COMMON_H
+#define SENTINEL_HIP_FLASH_COMMON_H
+
+#include <hip/hip_runtime.h>
+
+namespace sentinel_hip {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Problem geometry common to every kernel.
+struct AttnGeom {
+    int q_heads;
+    int kv_heads;
+    int head_dim;
+    int seq_len;
+    int packs;
+    float scale;
+    int causal;
+};
+
+// element(pack, head, t, c) = base[pack * pack_stride + head * head_stride + t * t_stride + c * c_stride]
+// Sentinel's column layout: pack_stride = seq_len, head_stride = head_dim * stride_columns, t_stride = 1,
+// c_stride = stride_columns (base already advanced by column_start).
+// [B,H,T,d]: pack_stride = heads * T * d, head_stride = T * d, t_stride = d, c_stride = 1.
+struct TensorMap {
+    long long pack_stride;
+    long long head_stride;
+    long long t_stride;
+    long long c_stride;
+};
+
+// row(pack, head, t) = base[pack * pack_stride + head * head_stride + t]   (lse, delta)
+struct RowMap {
+    long long pack_stride;
+    long long head_stride;
+};
+
+enum class Elem : int { F32 = 0, BF16 = 1, F16 = 2 };
+
+// ---- fp32 FMA path (flash_fp32.hip): any head_dim <= 128, any layout ----
+hipError_t launch_fwd_f32(const float* q, const float* k, const float* v, float* out, float* lse, TensorMap qm,
+                          TensorMap kvm, RowMap lm, AttnGeom g, hipStream_t stream);
+hipError_t launch_bwd_f32(const float* q, const float* k, const float* v, const float* out, const float* lse,
+                          const float* d_out, float* dq, float* dk, float* dv, float* delta, TensorMap qm, TensorMap kvm,
+                          RowMap lm, AttnGeom g, hipStream_t stream);
+
+// ---- MFMA path (flash_mfma_*.hip): bf16 / fp16 [B,H,T,d] tensors, head_dim 64 or 128 ----
+bool mfma_supported(int head_dim);
+// lse rows are addressed through `lm`; delta is q_heads x (packs * seq_len)
+hipError_t launch_fwd_mfma(Elem type, const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm,
+                           AttnGeom g, hipStream_t stream);
+hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* v, const void* out, const float* lse,
+                           RowMap lm, const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g,
+                           hipStream_t stream);
+
+// ---- layout adapter (layout_adapter.hip): Sentinel column layout fp32 <-> [B,H,T,d] bf16 / fp16 ----
+hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int heads, int head_dim, int stride_columns,
+                                  int seq_len, int packs, hipStream_t stream);
+hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,
+                                  int seq_len, int packs, hipStream_t stream);
+
+}  // namespace sentinel_hip
+#endif

@@ -1,0 +1,237 @@
+// Causal flash-attention forward on gfx950 matrix cores (bf16 / fp16 operands, fp32 accumulation).
+//
+// Replaces CudaFlashAttentionForwardWmma64Entry (sentinel/NeuralNet/Cuda/CudaFlashAttention.cu:1105-1266):
+// same result (O and per-query LSE = max + ln(sum), natural log of the scaled scores), different design:
+//   * tensors are [B, H, T, D] 16-bit, so every global access is a coalesced 128-bit (K, Q) or
+//     full-row dword (V) load; nothing is converted or gathered per tile;
+//   * a workgroup of 4 wavefronts owns 128 queries (32 per wavefront) and walks 64-key tiles;
+//     Q stays in registers for the whole kernel, K and V^T tiles are double-buffered in LDS and the
+//     next tile's global loads are in flight while the current one is multiplied;
+//   * S^T = K Q^T, so a lane owns one query: the online-softmax max / sum are in-register plus one
+//     v_permlane32_swap, and P^T feeds the P V product from registers (no LDS round trip);
+//   * key tiles above the diagonal are skipped; only tiles that cross it are masked;
+//   * grouped-query attention reads the shared K/V head in place.
+#include "flash_common.h"
+#include "mfma_tile.h"
+
+namespace sentinel_hip {
+namespace {
+
+constexpr int kFwdThreads = 256;
+constexpr int kFwdQueryTile = 128;
+constexpr int kFwdKeyTile = 64;
+
+template <typename E, int D, bool CAUSAL>
+__global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned short* __restrict__ q,
+                                                                   const unsigned short* __restrict__ k,
+                                                                   const unsigned short* __restrict__ v,
+                                                                   unsigned short* __restrict__ out,
+                                                                   float* __restrict__ lse, RowMap lm, AttnGeom g,
+                                                                   int q_tiles, int total_tiles) {
+    constexpr int KT = kFwdKeyTile;
+    typedef RowTile<KT, D, kFwdThreads> KTile;
+    typedef TransposedTile<KT, D, kFwdThreads> VTile;
+    constexpr int KS = KTile::kStride;
+    constexpr int VS = VTile::kStride;
+    constexpr int KSTEPS = D / 16;  // k-steps of the S^T product
+    constexpr int CB = D / 32;      // 32-row blocks of O^T
+
+    __shared__ __attribute__((aligned(16))) unsigned short k_lds[2][KT * KS];
+    __shared__ __attribute__((aligned(16))) unsigned short v_lds[2][D * VS];
+
+    // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of tiles so
+    // that the q-tiles of one head (which stream the same K/V) share one L2.
+    const int per_xcd = (int)gridDim.x / 8;
+    const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
+    if (tile_id >= total_tiles) return;
+    const int bh = tile_id / q_tiles;
+    const int qt = q_tiles - 1 - tile_id % q_tiles;  // longest first within a head
+    const int b = bh / g.q_heads;
+    const int h = bh % g.q_heads;
+    const int kvh = h / (g.q_heads / g.kv_heads);
+    const int T = g.seq_len;
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64;
+    const int lane = tid % 64;
+    const int n = lane % 32;
+    const int gh = lane / 32;
+
+    const unsigned short* qb = q + ((long long)b * g.q_heads + h) * T * D;
+    const unsigned short* kb = k + ((long long)b * g.kv_heads + kvh) * T * D;
+    const unsigned short* vb = v + ((long long)b * g.kv_heads + kvh) * T * D;
+
+    const int q0w = qt * kFwdQueryTile + wave * 32;  // first query of this wavefront
+    const int qrow = q0w + n;
+    const int qload = qrow < T ? qrow : T - 1;
+
+    // Q^T as B operand: column = query, contraction over head dims
+    u32x4 qf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+        qf[ks] = *reinterpret_cast<const u32x4*>(qb + (long long)qload * D + ks * 16 + gh * 8);
+
+    const int q_hi = min(T, (qt + 1) * kFwdQueryTile);        // one past the last query of the tile
+    const int kv_tiles = CAUSAL ? (q_hi + KT - 1) / KT : (T + KT - 1) / KT;
+
+    KTile kt;
+    VTile vt;
+    kt.load(kb, 0, T, tid);
+    vt.load(vb, 0, T, tid);
+    kt.store(k_lds[0], tid);
+    vt.store(v_lds[0], tid);
+    __syncthreads();
+
+    f32x16 acc[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[cb][i] = 0.0f;
+    float m_run = -__builtin_inff();
+    float l_run = 0.0f;  // this lane's half of the row sum
+    const float c2 = g.scale * kLog2e;
+
+    const int k_off = row_perm(n) * KS + gh * 8;  // K operand read: row carried by D row n
+    const int v_off = n * VS + gh * 8;            // V^T operand read
+
+    for (int j = 0; j < kv_tiles; ++j) {
+        const int buf = j & 1;
+        const bool more = j + 1 < kv_tiles;
+        if (more) {
+            kt.load(kb, (j + 1) * KT, T, tid);
+            vt.load(vb, (j + 1) * KT, T, tid);
+        }
+
+        const int key0 = j * KT;
+        // wavefront-uniform: the whole tile lies above this wavefront's diagonal
+        const bool skip = CAUSAL && key0 > q0w + 31;
+        if (!skip) {
+            f32x16 s[2];
+#pragma unroll
+            for (int kbk = 0; kbk < 2; ++kbk) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[kbk][i] = 0.0f;
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks) {
+                    const u32x4 a = lds_read128(&k_lds[buf][kbk * 32 * KS + k_off + ks * 16]);
+                    s[kbk] = E::mfma(a, qf[ks], s[kbk]);
+                }
+            }
+
+            const bool need_mask = (CAUSAL && key0 + KT - 1 > q0w) || (!CAUSAL && key0 + KT > T);
+            if (need_mask) {
+#pragma unroll
+                for (int kbk = 0; kbk < 2; ++kbk)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int key = key0 + kbk * 32 + perm_row_of_reg(i, gh);
+                        const bool dead = CAUSAL ? key > qrow : key >= T;
+                        if (dead) s[kbk][i] = -__builtin_inff();
+                    }
+            }
+
+            float mx = s[0][0];
+#pragma unroll
+            for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[0][i]);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[1][i]);
+            mx = half_max(mx);
+            const float m_new = fmaxf(m_run, mx);
+            const float mc = m_new * c2;
+            const float alpha = __builtin_amdgcn_exp2f(m_run * c2 - mc);
+
+            float psum = 0.0f;
+            u32x4 pf[4];  // P^T as B operand, four 16-key k-steps
+#pragma unroll
+            for (int kbk = 0; kbk < 2; ++kbk) {
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kbk][half * 8 + 2 * e], c2, -mc));
+                        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kbk][half * 8 + 2 * e + 1], c2, -mc));
+                        psum += p0 + p1;
+                        pf[kbk * 2 + half][e] = E::pack2(p0, p1);
+                    }
+                }
+            }
+            l_run = l_run * alpha + psum;
+            if (__any(m_new > m_run)) {
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[cb][i] *= alpha;
+            }
+            m_run = m_new;
+
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const u32x4 a = lds_read128(&v_lds[buf][cb * 32 * VS + v_off + c4 * 16]);
+                    acc[cb] = E::mfma(a, pf[c4], acc[cb]);
+                }
+            }
+        }
+
+        if (more) {
+            kt.store(k_lds[buf ^ 1], tid);
+            vt.store(v_lds[buf ^ 1], tid);
+        }
+        __syncthreads();
+    }
+
+    const float l_tot = half_sum(l_run);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if (qrow < T) {
+        unsigned short* op = out + ((long long)b * g.q_heads + h) * T * D + (long long)qrow * D;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                u32x2 w;
+                w[0] = E::pack2(acc[cb][a * 4 + 0] * inv, acc[cb][a * 4 + 1] * inv);
+                w[1] = E::pack2(acc[cb][a * 4 + 2] * inv, acc[cb][a * 4 + 3] * inv);
+                *reinterpret_cast<u32x2*>(op + cb * 32 + a * 8 + gh * 4) = w;
+            }
+        if (gh == 0)
+            lse[b * lm.pack_stride + h * lm.head_stride + qrow] = m_run * g.scale + (l_tot > 0.0f ? __logf(l_tot) : 0.0f);
+    }
+}
+
+template <typename E, int D>
+hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm, AttnGeom g,
+                   hipStream_t stream) {
+    const int q_tiles = (g.seq_len + kFwdQueryTile - 1) / kFwdQueryTile;
+    const int total = g.packs * g.q_heads * q_tiles;
+    const int grid = (total + 7) / 8 * 8;
+    auto qp = static_cast<const unsigned short*>(q);
+    auto kp = static_cast<const unsigned short*>(k);
+    auto vp = static_cast<const unsigned short*>(v);
+    auto op = static_cast<unsigned short*>(out);
+    if (g.causal)
+        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, true>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm,
+                           g, q_tiles, total);
+    else
+        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, false>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm,
+                           g, q_tiles, total);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool mfma_supported(int head_dim) { return head_dim == 64 || head_dim == 128; }
+
+hipError_t launch_fwd_mfma(Elem type, const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm,
+                           AttnGeom g, hipStream_t stream) {
+    if (type == Elem::BF16) {
+        if (g.head_dim == 64) return run_fwd<Bf16, 64>(q, k, v, out, lse, lm, g, stream);
+        if (g.head_dim == 128) return run_fwd<Bf16, 128>(q, k, v, out, lse, lm, g, stream);
+    } else if (type == Elem::F16) {
+        if (g.head_dim == 64) return run_fwd<Fp16, 64>(q, k, v, out, lse, lm, g, stream);
+        if (g.head_dim == 128) return run_fwd<Fp16, 128>(q, k, v, out, lse, lm, g, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace sentinel_hip

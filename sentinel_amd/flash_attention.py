@@ -1,0 +1,242 @@
+"""Host-side mirror of Sentinel's ``CudaFlashAttention`` over the HIP C ABI.
+
+``HipFlashAttention`` keeps the names, argument order and error behaviour of
+``class CudaFlashAttention`` (sentinel/NeuralNet/Cuda/CudaFlashAttention.hpp:12-41): matrices are
+``(head_count * head_dimension) x columns`` fp32 device tensors, the column window / pack arguments mean
+the same, shape errors raise ``ValueError`` (std::invalid_argument there) and device / launch errors raise
+``RuntimeError``.  torch is used only to own device memory and to name the stream; all arithmetic runs in
+``libsentinel_hip_attn.so`` and nothing here falls back to another implementation: a missing library is an
+error.
+
+``flash_attention_forward`` / ``flash_attention_backward`` are the native entry points on contiguous
+``[B, H, T, d]`` bf16 / fp16 (or fp32) tensors.
+"""
+import ctypes
+import math
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "lib", "libsentinel_hip_attn.so")
+
+OK, INVALID_ARGUMENT, UNSUPPORTED, RUNTIME = 0, 1, 2, 3
+F32, BF16, F16 = 0, 1, 2
+COMPUTE_AUTO = -1
+LAYOUT_COLUMNS, LAYOUT_BHTD = 0, 1
+
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+_COMPUTE_CODE = {None: COMPUTE_AUTO, "auto": COMPUTE_AUTO, "fp32": F32, "bf16": BF16, "fp16": F16,
+                 torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+
+_lib = None
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def load_library():
+    """Load the built HIP library; raises if it has not been built (python -m sentinel_amd.build)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise ImportError(f"{_LIB_PATH} is missing: build it with `python -m sentinel_amd.build` "
+                          "(there is no fallback implementation)")
+    lib = ctypes.CDLL(_LIB_PATH)
+    vp, i, f, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+    lib.sentinel_hip_flash_fwd.argtypes = [vp] * 5 + [i] * 10 + [f, i, vp, sz, vp]
+    lib.sentinel_hip_flash_fwd.restype = i
+    lib.sentinel_hip_flash_bwd.argtypes = [vp] * 10 + [i] * 10 + [f, i, vp, sz, vp]
+    lib.sentinel_hip_flash_bwd.restype = i
+    lib.sentinel_hip_flash_workspace_bytes.argtypes = [i] * 9
+    lib.sentinel_hip_flash_workspace_bytes.restype = sz
+    lib.sentinel_hip_flash_max_head_dim.restype = i
+    lib.sentinel_hip_device_available.restype = i
+    lib.sentinel_hip_strerror.argtypes = [i]
+    lib.sentinel_hip_strerror.restype = ctypes.c_char_p
+    lib.sentinel_hip_last_error.restype = ctypes.c_char_p
+    _lib = lib
+    return lib
+
+
+def _check(code):
+    if code == OK:
+        return
+    lib = load_library()
+    detail = lib.sentinel_hip_last_error().decode() or lib.sentinel_hip_strerror(code).decode()
+    if code in (INVALID_ARGUMENT, UNSUPPORTED):
+        raise ValueError(detail)
+    raise RuntimeError(detail)
+
+
+def _stream_handle(stream):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _ensure_size(t, rows, cols, like):
+    """CudaMatrix::ensureSize for an optional output tensor."""
+    if t is None or tuple(t.shape) != (rows, cols):
+        return torch.empty((rows, cols), dtype=torch.float32, device=like.device)
+    return t
+
+
+def _workspace(lib, io, compute, layout, hq, hkv, d, t, packs, backward, device, workspace):
+    need = lib.sentinel_hip_flash_workspace_bytes(io, compute, layout, hq, hkv, d, t, packs, int(backward))
+    if need == 0:
+        return None, 0
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=device)
+    return workspace, need
+
+
+class HipFlashAttention:
+    """Static interface of Sentinel's CudaFlashAttention on MI355X."""
+
+    query_tile_size = 128
+    key_tile_size = 64
+    max_head_dimension = 128
+
+    @staticmethod
+    def forward_multi_head(query, key, value, out, log_sum_exp, head_count, head_dimension, scale, causal=True,
+                           column_start=0, column_count=0, pack_count=1, *, kv_head_count=None, compute=None,
+                           workspace=None, stream=None):
+        """CudaFlashAttention::forwardMultiHead. Returns (out, log_sum_exp) (re-allocated if their shape was wrong)."""
+        lib = load_library()
+        HipFlashAttention._validate(query, key, value, head_count, head_dimension, kv_head_count, "forwardMultiHead")
+        kv_heads = head_count if kv_head_count in (None, 0) else kv_head_count
+        rows, cols = query.shape
+        out = _ensure_size(out, rows, cols, query)
+        log_sum_exp = _ensure_size(log_sum_exp, head_count, cols, query)
+        comp = _COMPUTE_CODE[compute]
+        seq = column_count if column_count > 0 else cols - column_start
+        ws, ws_bytes = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1),
+                                  max(pack_count, 1), False, query.device, workspace)
+        _check(lib.sentinel_hip_flash_fwd(_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp), F32, comp,
+                                          LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start,
+                                          column_count, pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes,
+                                          _stream_handle(stream)))
+        return out, log_sum_exp
+
+    @staticmethod
+    def forward(query, key, value, out, log_sum_exp, scale, causal=True, **kw):
+        """CudaFlashAttention::forward: single head, head_dimension = rows."""
+        return HipFlashAttention.forward_multi_head(query, key, value, out, log_sum_exp, 1, int(query.shape[0]), scale,
+                                                    causal, 0, int(query.shape[1]), 1, **kw)
+
+    @staticmethod
+    def backward_multi_head(query, key, value, out, log_sum_exp, out_gradient, query_gradient, key_gradient,
+                            value_gradient, delta_workspace, head_count, head_dimension, scale, causal=True,
+                            column_start=0, column_count=0, pack_count=1, *, kv_head_count=None, compute=None,
+                            workspace=None, stream=None):
+        """CudaFlashAttention::backwardMultiHead. Returns (dQ, dK, dV, delta)."""
+        lib = load_library()
+        HipFlashAttention._validate(query, key, value, head_count, head_dimension, kv_head_count, "backwardMultiHead")
+        kv_heads = head_count if kv_head_count in (None, 0) else kv_head_count
+        rows, cols = query.shape
+        if tuple(out.shape) != (rows, cols):
+            raise ValueError("HipFlashAttention::backwardMultiHead out shape mismatch")
+        if tuple(out_gradient.shape) != (rows, cols):
+            raise ValueError("HipFlashAttention::backwardMultiHead outGradient shape mismatch")
+        if tuple(log_sum_exp.shape) != (head_count, cols):
+            raise ValueError("HipFlashAttention::backwardMultiHead logSumExp shape mismatch")
+        seq = column_count if column_count > 0 else cols - column_start
+        packs = max(pack_count, 1)
+        query_gradient = _ensure_size(query_gradient, rows, cols, query)
+        key_gradient = _ensure_size(key_gradient, key.shape[0], cols, query)
+        value_gradient = _ensure_size(value_gradient, value.shape[0], cols, query)
+        delta_workspace = _ensure_size(delta_workspace, head_count, packs * max(seq, 1), query)
+        comp = _COMPUTE_CODE[compute]
+        ws, ws_bytes = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1), packs,
+                                  True, query.device, workspace)
+        _check(lib.sentinel_hip_flash_bwd(_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp),
+                                          _ptr(out_gradient), _ptr(query_gradient), _ptr(key_gradient),
+                                          _ptr(value_gradient), _ptr(delta_workspace), F32, comp, LAYOUT_COLUMNS,
+                                          head_count, kv_heads, head_dimension, cols, column_start, column_count,
+                                          pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes,
+                                          _stream_handle(stream)))
+        return query_gradient, key_gradient, value_gradient, delta_workspace
+
+    @staticmethod
+    def backward(query, key, value, out, log_sum_exp, out_gradient, query_gradient, key_gradient, value_gradient, scale,
+                 causal=True, **kw):
+        """CudaFlashAttention::backward: single head."""
+        return HipFlashAttention.backward_multi_head(query, key, value, out, log_sum_exp, out_gradient, query_gradient,
+                                                     key_gradient, value_gradient, None, 1, int(query.shape[0]), scale,
+                                                     causal, 0, int(query.shape[1]), 1, **kw)[:3]
+
+    @staticmethod
+    def _validate(query, key, value, head_count, head_dimension, kv_head_count, op):
+        # validateMultiHeadShape (CudaFlashAttention.cu:1458-1471), with the K/V rows rule widened to grouped heads
+        name = f"HipFlashAttention::{op}"
+        for t in (query, key, value):
+            if t is None or t.dim() != 2 or t.numel() == 0:
+                raise ValueError(f"{name} empty input")
+            if t.dtype != torch.float32 or not t.is_contiguous():
+                raise ValueError(f"{name} expects contiguous fp32 matrices")
+        if head_count <= 0 or head_dimension <= 0:
+            raise ValueError(f"{name} invalid head geometry")
+        if head_dimension > HipFlashAttention.max_head_dimension:
+            raise ValueError(f"{name} headDim exceeds maxHeadDimension")
+        kv_heads = head_count if kv_head_count in (None, 0) else kv_head_count
+        if kv_heads <= 0 or head_count % kv_heads != 0:
+            raise ValueError(f"{name} headCount must be divisible by kvHeadCount")
+        if query.shape[0] != head_count * head_dimension:
+            raise ValueError(f"{name} query rows mismatch headCount*headDim")
+        if key.shape[0] != kv_heads * head_dimension or value.shape[0] != key.shape[0]:
+            raise ValueError(f"{name} key/value rows mismatch")
+        if query.shape[1] != key.shape[1] or query.shape[1] != value.shape[1]:
+            raise ValueError(f"{name} sequenceLength mismatch")
+        if not load_library().sentinel_hip_device_available():
+            raise RuntimeError(f"{name} no HIP device")
+
+
+def _bhtd_geometry(q, k, v):
+    if q.dim() != 4 or k.dim() != 4 or v.shape != k.shape:
+        raise ValueError("flash_attention expects [B, H, T, d] tensors")
+    b, hq, t, d = q.shape
+    if k.shape[0] != b or k.shape[2] != t or k.shape[3] != d:
+        raise ValueError("flash_attention q / k shape mismatch")
+    for x in (q, k, v):
+        if not x.is_contiguous() or x.dtype != q.dtype:
+            raise ValueError("flash_attention expects contiguous tensors of one dtype")
+    if q.dtype not in _DTYPE_CODE:
+        raise ValueError(f"flash_attention unsupported dtype {q.dtype}")
+    return b, hq, k.shape[1], t, d
+
+
+def flash_attention_forward(q, k, v, scale=None, causal=True, out=None, lse=None, stream=None):
+    """Native forward on [B,H,T,d] tensors (k, v may have fewer heads). Returns (out, lse[B,H,T] fp32)."""
+    lib = load_library()
+    b, hq, hkv, t, d = _bhtd_geometry(q, k, v)
+    scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
+    out = torch.empty_like(q) if out is None else out
+    lse = torch.empty((b, hq, t), dtype=torch.float32, device=q.device) if lse is None else lse
+    code = _DTYPE_CODE[q.dtype]
+    _check(lib.sentinel_hip_flash_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), code, COMPUTE_AUTO, LAYOUT_BHTD, hq,
+                                      hkv, d, 0, 0, t, b, scale, int(bool(causal)), None, 0, _stream_handle(stream)))
+    return out, lse
+
+
+def flash_attention_backward(q, k, v, out, lse, d_out, scale=None, causal=True, dq=None, dk=None, dv=None, delta=None,
+                             stream=None):
+    """Native backward on [B,H,T,d] tensors. Returns (dq, dk, dv)."""
+    lib = load_library()
+    b, hq, hkv, t, d = _bhtd_geometry(q, k, v)
+    scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
+    dq = torch.empty_like(q) if dq is None else dq
+    dk = torch.empty_like(k) if dk is None else dk
+    dv = torch.empty_like(v) if dv is None else dv
+    delta = torch.empty((hq, b * t), dtype=torch.float32, device=q.device) if delta is None else delta
+    code = _DTYPE_CODE[q.dtype]
+    _check(lib.sentinel_hip_flash_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out), _ptr(dq), _ptr(dk),
+                                      _ptr(dv), _ptr(delta), code, COMPUTE_AUTO, LAYOUT_BHTD, hq, hkv, d, 0, 0, t, b, scale,
+                                      int(bool(causal)), None, 0, _stream_handle(stream)))
+    return dq, dk, dv
