@@ -74,13 +74,26 @@ __device__ __forceinline__ int perm_row_of_reg(int i, int g) { return ((i >> 3) 
 __device__ __forceinline__ int plain_row_of_reg(int i, int g) { return ((i >> 2) << 3) | (g << 2) | (i & 3); }
 
 // max / sum across the two lane halves (lane n <-> lane n+32); every lane gets the combined value.
+// v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second:
+// starting from two copies of x, the first ends up holding lane n's x in lanes n and n+32, the second
+// lane n+32's x in both.  Written as inline assembly because the compiler builtin returns its first
+// result twice; the s_nop covers the VALU-write -> permlane-read wait states the assembler cannot see.
+__device__ __forceinline__ void half_exchange(float x, float& from_low, float& from_high) {
+    float a = x;
+    float b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    from_low = a;
+    from_high = b;
+}
 __device__ __forceinline__ float half_max(float x) {
-    auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
-    return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+    float lo, hi;
+    half_exchange(x, lo, hi);
+    return fmaxf(lo, hi);
 }
 __device__ __forceinline__ float half_sum(float x) {
-    auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
-    return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
+    float lo, hi;
+    half_exchange(x, lo, hi);
+    return lo + hi;
 }
 
 __device__ __forceinline__ u32x4 lds_read128(const unsigned short* p) { return *reinterpret_cast<const u32x4*>(p); }
