@@ -1,7 +1,520 @@
+// Causal flash-attention backward on gfx950 matrix cores (bf16 / fp16 operands, fp32 accumulation).
+//
+// Replaces CudaFlashAttentionDeltaEntry + CudaFlashAttentionBackwardQueryWmma64Entry
+// (sentinel/NeuralNet/Cuda/CudaFlashAttention.cu:576-596, :1269-1456).  Same mathematics
+//     P = exp(S - LSE),  dP = dO V^T,  dS = P o (dP - D) * scale,
+//     dV = P^T dO,  dK = dS^T Q,  dQ = dS K,          D = rowsum(dO o O)
+// but no atomics and no pre-zeroed outputs: the work is split into
+//   delta_mfma_kernel   D per query;
+//   dkdv_mfma_kernel    key-outer: a workgroup owns 128 keys of one K/V head, keeps K, V (as B operands)
+//                       and the dK^T, dV^T accumulators in registers, and streams the query tiles of every
+//                       query head of the group through LDS (grouped-query gradients are summed in
+//                       registers, replacing reduceKvHeadGradsInto, CudaCausalSelfAttention.cu:36-44);
+//   dq_mfma_kernel      query-outer: a workgroup owns 128 queries, keeps Q, dO (as B operands) and dQ^T in
+//                       registers and streams K / V tiles through LDS (recomputing S and dP).
+// In both kernels the score-like tiles are produced so that one lane owns one key (dK/dV kernel) or one
+// query (dQ kernel) and their registers are, after type conversion, directly the B operand of the
+// following product (see mfma_tile.h).
 #include "flash_common.h"
+#include "mfma_tile.h"
+
 namespace sentinel_hip {
-hipError_t launch_bwd_mfma(Elem, const void*, const void*, const void*, const void*, const float*, RowMap, const void*, void*,
-                           void*, void*, float*, AttnGeom, hipStream_t) {
-    return hipErrorNotSupported;
+namespace {
+
+constexpr int kBwdThreads = 256;
+
+// ------------------------------------------------------------------------------------------------
+// D[h][b*T + t] = sum_c out * d_out  (16-bit inputs, fp32 sum)
+// ------------------------------------------------------------------------------------------------
+template <typename E, int D>
+__global__ __launch_bounds__(kBwdThreads) void delta_mfma_kernel(const unsigned short* __restrict__ out,
+                                                                  const unsigned short* __restrict__ d_out,
+                                                                  float* __restrict__ delta, AttnGeom g) {
+    constexpr int LPR = D / 8;  // lanes per row
+    constexpr int RPB = kBwdThreads / LPR;
+    const int tid = threadIdx.x;
+    const int row = blockIdx.x * RPB + tid / LPR;
+    const int part = tid % LPR;
+    const int h = blockIdx.y;
+    const int b = blockIdx.z;
+    const int T = g.seq_len;
+    float sum = 0.0f;
+    if (row < T) {
+        const long long off = (((long long)b * g.q_heads + h) * T + row) * D + part * 8;
+        const u32x4 o = *reinterpret_cast<const u32x4*>(out + off);
+        const u32x4 d = *reinterpret_cast<const u32x4*>(d_out + off);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sum += E::lo(o[e]) * E::lo(d[e]) + E::hi(o[e]) * E::hi(d[e]);
+    }
+#pragma unroll
+    for (int step = LPR / 2; step >= 1; step /= 2) sum += __shfl_xor(sum, step, LPR);
+    if (part == 0 && row < T) delta[(long long)h * g.packs * T + (long long)b * T + row] = sum;
 }
+
+// ------------------------------------------------------------------------------------------------
+// dQ: query-outer
+// ------------------------------------------------------------------------------------------------
+constexpr int kDqQueryTile = 128;
+constexpr int kDqKeyTile = 64;
+
+template <typename E, int D, bool CAUSAL>
+__global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dq_mfma_kernel(const unsigned short* __restrict__ q,
+                                                                  const unsigned short* __restrict__ k,
+                                                                  const unsigned short* __restrict__ v,
+                                                                  const unsigned short* __restrict__ d_out,
+                                                                  const float* __restrict__ lse,
+                                                                  const float* __restrict__ delta,
+                                                                  unsigned short* __restrict__ dq, RowMap lm, AttnGeom g,
+                                                                  int q_tiles, int total_tiles) {
+    constexpr int KT = kDqKeyTile;
+    typedef RowTile<KT, D, kBwdThreads> RTile;
+    typedef TransposedTile<KT, D, kBwdThreads> TTile;
+    constexpr int KS = RTile::kStride;
+    constexpr int TS = TTile::kStride;
+    constexpr int KSTEPS = D / 16;
+    constexpr int CB = D / 32;
+
+    __shared__ __attribute__((aligned(16))) unsigned short k_lds[KT * KS];
+    __shared__ __attribute__((aligned(16))) unsigned short v_lds[KT * KS];
+    __shared__ __attribute__((aligned(16))) unsigned short kt_lds[D * TS];
+
+    const int per_xcd = (int)gridDim.x / 8;
+    const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
+    if (tile_id >= total_tiles) return;
+    const int bh = tile_id / q_tiles;
+    const int qt = q_tiles - 1 - tile_id % q_tiles;
+    const int b = bh / g.q_heads;
+    const int h = bh % g.q_heads;
+    const int kvh = h / (g.q_heads / g.kv_heads);
+    const int T = g.seq_len;
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64;
+    const int lane = tid % 64;
+    const int n = lane % 32;
+    const int gh = lane / 32;
+
+    const long long q_head = ((long long)b * g.q_heads + h) * T * D;
+    const unsigned short* kb = k + ((long long)b * g.kv_heads + kvh) * T * D;
+    const unsigned short* vb = v + ((long long)b * g.kv_heads + kvh) * T * D;
+
+    const int q0w = qt * kDqQueryTile + wave * 32;
+    const int qrow = q0w + n;
+    const int qload = qrow < T ? qrow : T - 1;
+
+    u32x4 qf[KSTEPS];
+    u32x4 gf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        qf[ks] = *reinterpret_cast<const u32x4*>(q + q_head + (long long)qload * D + ks * 16 + gh * 8);
+        gf[ks] = *reinterpret_cast<const u32x4*>(d_out + q_head + (long long)qload * D + ks * 16 + gh * 8);
+    }
+    const float c2 = g.scale * kLog2e;
+    const float lse2 = lse[b * lm.pack_stride + h * lm.head_stride + qload] * kLog2e;
+    const float dl = delta[(long long)h * g.packs * T + (long long)b * T + qload];
+
+    const int q_hi = min(T, (qt + 1) * kDqQueryTile);
+    const int kv_tiles = CAUSAL ? (q_hi + KT - 1) / KT : (T + KT - 1) / KT;
+
+    RTile ktile;
+    RTile vtile;
+    TTile kttile;
+    ktile.load(kb, 0, T, tid);
+    vtile.load(vb, 0, T, tid);
+    kttile.load(kb, 0, T, tid);
+    ktile.store(k_lds, tid);
+    vtile.store(v_lds, tid);
+    kttile.store(kt_lds, tid);
+    __syncthreads();
+
+    f32x16 acc[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[cb][i] = 0.0f;
+
+    const int k_off = row_perm(n) * KS + gh * 8;
+    const int t_off = n * TS + gh * 8;
+
+    for (int j = 0; j < kv_tiles; ++j) {
+        const bool more = j + 1 < kv_tiles;
+        if (more) {
+            ktile.load(kb, (j + 1) * KT, T, tid);
+            vtile.load(vb, (j + 1) * KT, T, tid);
+            kttile.load(kb, (j + 1) * KT, T, tid);
+        }
+        const int key0 = j * KT;
+        const bool skip = CAUSAL && key0 > q0w + 31;
+        if (!skip) {
+            f32x16 s[2];
+            f32x16 dp[2];
+#pragma unroll
+            for (int kbk = 0; kbk < 2; ++kbk) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s[kbk][i] = 0.0f;
+                    dp[kbk][i] = 0.0f;
+                }
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks) {
+                    const u32x4 ak = lds_read128(&k_lds[kbk * 32 * KS + k_off + ks * 16]);
+                    s[kbk] = E::mfma(ak, qf[ks], s[kbk]);
+                    const u32x4 av = lds_read128(&v_lds[kbk * 32 * KS + k_off + ks * 16]);
+                    dp[kbk] = E::mfma(av, gf[ks], dp[kbk]);
+                }
+            }
+            const bool need_mask = CAUSAL ? (key0 + KT - 1 > q0w) : (key0 + KT > T);
+            u32x4 dsf[4];
+#pragma unroll
+            for (int kbk = 0; kbk < 2; ++kbk) {
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float ds2[2];
+#pragma unroll
+                        for (int w = 0; w < 2; ++w) {
+                            const int i = half * 8 + 2 * e + w;
+                            float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kbk][i], c2, -lse2));
+                            if (need_mask) {
+                                const int key = key0 + kbk * 32 + perm_row_of_reg(i, gh);
+                                const bool dead = CAUSAL ? key > qrow : key >= T;
+                                if (dead) p = 0.0f;
+                            }
+                            ds2[w] = p * (dp[kbk][i] - dl);
+                        }
+                        dsf[kbk * 2 + half][e] = E::pack2(ds2[0], ds2[1]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const u32x4 a = lds_read128(&kt_lds[cb * 32 * TS + t_off + c4 * 16]);
+                    acc[cb] = E::mfma(a, dsf[c4], acc[cb]);
+                }
+            }
+        }
+        __syncthreads();
+        if (more) {
+            ktile.store(k_lds, tid);
+            vtile.store(v_lds, tid);
+            kttile.store(kt_lds, tid);
+        }
+        __syncthreads();
+    }
+
+    if (qrow < T) {
+        unsigned short* dst = dq + q_head + (long long)qrow * D;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                u32x2 w;
+                w[0] = E::pack2(acc[cb][a * 4 + 0] * g.scale, acc[cb][a * 4 + 1] * g.scale);
+                w[1] = E::pack2(acc[cb][a * 4 + 2] * g.scale, acc[cb][a * 4 + 3] * g.scale);
+                *reinterpret_cast<u32x2*>(dst + cb * 32 + a * 8 + gh * 4) = w;
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// dK, dV: key-outer
+// ------------------------------------------------------------------------------------------------
+constexpr int kDkvKeyTile = 128;
+constexpr int kDkvQueryTile = 64;
+
+template <int D>
+struct DkvLds {
+    static constexpr int QT = kDkvQueryTile;
+    static constexpr int QS = D + 8;
+    static constexpr int TS = QT + 8;
+    unsigned short q[QT * QS];
+    unsigned short g[QT * QS];
+    unsigned short qt[D * TS];
+    unsigned short gt[D * TS];
+    float lse2[QT];
+    float dl[QT];
+};
+
+template <typename E, int D, bool CAUSAL>
+__global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kernel(
+    const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
+    const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
+    unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
+    int total_tiles) {
+    constexpr int QT = kDkvQueryTile;
+    typedef RowTile<QT, D, kBwdThreads> RTile;
+    typedef TransposedTile<QT, D, kBwdThreads> TTile;
+    constexpr int QS = RTile::kStride;
+    constexpr int TS = TTile::kStride;
+    static_assert(QS == DkvLds<D>::QS && TS == DkvLds<D>::TS, "LDS layout mismatch");
+    constexpr int KSTEPS = D / 16;
+    constexpr int CB = D / 32;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char dkv_smem[];
+    DkvLds<D>* lds = reinterpret_cast<DkvLds<D>*>(dkv_smem);  // two stages
+
+    const int per_xcd = (int)gridDim.x / 8;
+    const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
+    if (tile_id >= total_tiles) return;
+    const int bkv = tile_id / k_tiles;
+    const int ktile = tile_id % k_tiles;  // under the causal mask the first key tiles see the most queries
+    const int b = bkv / g.kv_heads;
+    const int kvh = bkv % g.kv_heads;
+    const int group = g.q_heads / g.kv_heads;
+    const int T = g.seq_len;
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64;
+    const int lane = tid % 64;
+    const int n = lane % 32;
+    const int gh = lane / 32;
+
+    const long long kv_head = ((long long)b * g.kv_heads + kvh) * T * D;
+    const int k0w = ktile * kDkvKeyTile + wave * 32;
+    const int key = k0w + n;
+    const int kload = key < T ? key : T - 1;
+    const bool key_dead = key >= T;
+
+    // K^T and V^T as B operands: column = key, contraction over head dims
+    u32x4 kf[KSTEPS];
+    u32x4 vf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        kf[ks] = *reinterpret_cast<const u32x4*>(k + kv_head + (long long)kload * D + ks * 16 + gh * 8);
+        vf[ks] = *reinterpret_cast<const u32x4*>(v + kv_head + (long long)kload * D + ks * 16 + gh * 8);
+    }
+    const float c2 = g.scale * kLog2e;
+
+    const int q_tiles_all = (T + QT - 1) / QT;
+    const int q_first = CAUSAL ? (ktile * kDkvKeyTile) / QT : 0;
+    const int n_qt = q_tiles_all - q_first;
+    const int n_iter = group * n_qt;
+
+    f32x16 dk_acc[CB];
+    f32x16 dv_acc[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            dk_acc[cb][i] = 0.0f;
+            dv_acc[cb][i] = 0.0f;
+        }
+
+    RTile qtile;
+    RTile gtile;
+    TTile qttile;
+    TTile gttile;
+    float row_val = 0.0f;  // threads 0..63: lse * log2(e); threads 64..127: delta
+
+    auto load_stage = [&](int it) {
+        const int h = kvh * group + it / n_qt;
+        const int q0 = (q_first + it % n_qt) * QT;
+        const long long q_head = ((long long)b * g.q_heads + h) * T * D;
+        qtile.load(q + q_head, q0, T, tid);
+        gtile.load(d_out + q_head, q0, T, tid);
+        qttile.load(q + q_head, q0, T, tid);
+        gttile.load(d_out + q_head, q0, T, tid);
+        if (tid < QT) {
+            const int t = q0 + tid;
+            row_val = t < T ? lse[b * lm.pack_stride + h * lm.head_stride + t] * kLog2e : __builtin_inff();
+        } else if (tid < 2 * QT) {
+            const int t = q0 + tid - QT;
+            row_val = t < T ? delta[(long long)h * g.packs * T + (long long)b * T + t] : 0.0f;
+        }
+    };
+    auto store_stage = [&](DkvLds<D>& st) {
+        qtile.store(st.q, tid);
+        gtile.store(st.g, tid);
+        qttile.store(st.qt, tid);
+        gttile.store(st.gt, tid);
+        if (tid < QT)
+            st.lse2[tid] = row_val;
+        else if (tid < 2 * QT)
+            st.dl[tid - QT] = row_val;
+    };
+
+    if (n_iter > 0) {
+        load_stage(0);
+        store_stage(lds[0]);
+    }
+    __syncthreads();
+
+    const int r_off = row_perm(n) * QS + gh * 8;
+    const int t_off = n * TS + gh * 8;
+
+    for (int it = 0; it < n_iter; ++it) {
+        const bool more = it + 1 < n_iter;
+        if (more) load_stage(it + 1);
+        DkvLds<D>& st = lds[it & 1];
+        const int q0 = (q_first + it % n_qt) * QT;
+
+#pragma unroll
+        for (int qb = 0; qb < QT / 32; ++qb) {
+            const int q0b = q0 + qb * 32;
+            const bool skip = (CAUSAL && q0b + 31 < k0w) || q0b >= T;
+            if (skip) continue;
+            f32x16 s;
+            f32x16 dp;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                s[i] = 0.0f;
+                dp[i] = 0.0f;
+            }
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                const u32x4 aq = lds_read128(&st.q[qb * 32 * QS + r_off + ks * 16]);
+                s = E::mfma(aq, kf[ks], s);
+                const u32x4 ag = lds_read128(&st.g[qb * 32 * QS + r_off + ks * 16]);
+                dp = E::mfma(ag, vf[ks], dp);
+            }
+            // per-query lse and delta of the 16 queries this lane holds: two runs of eight
+            float l2[16];
+            float dl[16];
+#pragma unroll
+            for (int run = 0; run < 2; ++run)
+#pragma unroll
+                for (int part = 0; part < 2; ++part) {
+                    const int base = qb * 32 + run * 16 + gh * 8 + part * 4;
+                    const float4 a = *reinterpret_cast<const float4*>(&st.lse2[base]);
+                    const float4 d4 = *reinterpret_cast<const float4*>(&st.dl[base]);
+                    const int i0 = run * 8 + part * 4;
+                    l2[i0] = a.x; l2[i0 + 1] = a.y; l2[i0 + 2] = a.z; l2[i0 + 3] = a.w;
+                    dl[i0] = d4.x; dl[i0 + 1] = d4.y; dl[i0 + 2] = d4.z; dl[i0 + 3] = d4.w;
+                }
+            const bool need_mask = CAUSAL && q0b < k0w + 31;
+            u32x4 pf[2];
+            u32x4 dsf[2];
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float p2[2];
+                    float ds2[2];
+#pragma unroll
+                    for (int w = 0; w < 2; ++w) {
+                        const int i = half * 8 + 2 * e + w;
+                        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -l2[i]));
+                        if (need_mask) {
+                            const int query = q0b + perm_row_of_reg(i, gh);
+                            if (key > query) p = 0.0f;
+                        }
+                        if (key_dead) p = 0.0f;
+                        p2[w] = p;
+                        ds2[w] = p * (dp[i] - dl[i]);
+                    }
+                    pf[half][e] = E::pack2(p2[0], p2[1]);
+                    dsf[half][e] = E::pack2(ds2[0], ds2[1]);
+                }
+            }
+#pragma unroll
+            for (int c2i = 0; c2i < 2; ++c2i) {
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const u32x4 ag = lds_read128(&st.gt[cb * 32 * TS + t_off + qb * 32 + c2i * 16]);
+                    dv_acc[cb] = E::mfma(ag, pf[c2i], dv_acc[cb]);
+                    const u32x4 aq = lds_read128(&st.qt[cb * 32 * TS + t_off + qb * 32 + c2i * 16]);
+                    dk_acc[cb] = E::mfma(aq, dsf[c2i], dk_acc[cb]);
+                }
+            }
+        }
+
+        if (more) store_stage(lds[(it + 1) & 1]);
+        __syncthreads();
+    }
+
+    if (!key_dead) {
+        unsigned short* dkp = dk + kv_head + (long long)key * D;
+        unsigned short* dvp = dv + kv_head + (long long)key * D;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                u32x2 wk, wv;
+                wk[0] = E::pack2(dk_acc[cb][a * 4 + 0] * g.scale, dk_acc[cb][a * 4 + 1] * g.scale);
+                wk[1] = E::pack2(dk_acc[cb][a * 4 + 2] * g.scale, dk_acc[cb][a * 4 + 3] * g.scale);
+                wv[0] = E::pack2(dv_acc[cb][a * 4 + 0], dv_acc[cb][a * 4 + 1]);
+                wv[1] = E::pack2(dv_acc[cb][a * 4 + 2], dv_acc[cb][a * 4 + 3]);
+                *reinterpret_cast<u32x2*>(dkp + cb * 32 + a * 8 + gh * 4) = wk;
+                *reinterpret_cast<u32x2*>(dvp + cb * 32 + a * 8 + gh * 4) = wv;
+            }
+    }
+}
+
+template <typename E, int D>
+hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse, RowMap lm,
+                   const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g, hipStream_t stream) {
+    auto qp = static_cast<const unsigned short*>(q);
+    auto kp = static_cast<const unsigned short*>(k);
+    auto vp = static_cast<const unsigned short*>(v);
+    auto op = static_cast<const unsigned short*>(out);
+    auto gp = static_cast<const unsigned short*>(d_out);
+    auto dqp = static_cast<unsigned short*>(dq);
+    auto dkp = static_cast<unsigned short*>(dk);
+    auto dvp = static_cast<unsigned short*>(dv);
+    const int T = g.seq_len;
+
+    constexpr int RPB = kBwdThreads / (D / 8);
+    hipLaunchKernelGGL((delta_mfma_kernel<E, D>), dim3((T + RPB - 1) / RPB, g.q_heads, g.packs), dim3(kBwdThreads), 0,
+                       stream, op, gp, delta, g);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+
+    // dK, dV
+    {
+        const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
+        const int total = g.packs * g.kv_heads * k_tiles;
+        const int grid = (total + 7) / 8 * 8;
+        const size_t smem = 2 * sizeof(DkvLds<D>);
+        static bool raised[2] = {false, false};  // one-time opt-in to more than 64 KiB of LDS per kernel
+        const int which = g.causal ? 1 : 0;
+        if (!raised[which]) {
+            const void* fn = g.causal ? reinterpret_cast<const void*>(dkdv_mfma_kernel<E, D, true>)
+                                      : reinterpret_cast<const void*>(dkdv_mfma_kernel<E, D, false>);
+            err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+            if (err != hipSuccess) return err;
+            raised[which] = true;
+        }
+        if (g.causal)
+            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, true>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp,
+                               lse, delta, dkp, dvp, lm, g, k_tiles, total);
+        else
+            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, false>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp,
+                               lse, delta, dkp, dvp, lm, g, k_tiles, total);
+        err = hipGetLastError();
+        if (err != hipSuccess) return err;
+    }
+    // dQ
+    {
+        const int q_tiles = (T + kDqQueryTile - 1) / kDqQueryTile;
+        const int total = g.packs * g.q_heads * q_tiles;
+        const int grid = (total + 7) / 8 * 8;
+        if (g.causal)
+            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp, lse,
+                               delta, dqp, lm, g, q_tiles, total);
+        else
+            hipLaunchKernelGGL((dq_mfma_kernel<E, D, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp, lse,
+                               delta, dqp, lm, g, q_tiles, total);
+        err = hipGetLastError();
+    }
+    return err;
+}
+
+}  // namespace
+
+hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* v, const void* out, const float* lse,
+                           RowMap lm, const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g,
+                           hipStream_t stream) {
+    if (type == Elem::BF16) {
+        if (g.head_dim == 64) return run_bwd<Bf16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, stream);
+        if (g.head_dim == 128) return run_bwd<Bf16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, stream);
+    } else if (type == Elem::F16) {
+        if (g.head_dim == 64) return run_bwd<Fp16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, stream);
+        if (g.head_dim == 128) return run_bwd<Fp16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
 }  // namespace sentinel_hip

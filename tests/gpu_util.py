@@ -48,10 +48,13 @@ def assert_close_fp32(got, want, name, tol=1e-4):
     assert worst <= 1.0, f"{name}: error {float(err.max()):.3e} exceeds {tol} (ratio {worst:.2f})"
 
 
-def assert_close_lowp(got, want, name, tol=2e-2):
-    """north-star bf16 / fp16 bar: 2e-2 relative, taken norm-wise: max|got - want| <= tol * max|want|"""
+def assert_close_lowp(got, want, name, tol=2e-2, floor=1e-5):
+    """north-star bf16 / fp16 bar: 2e-2 relative, taken norm-wise: max|got - want| <= tol * max|want| (+ floor).
+
+    The absolute floor only matters where the exact answer is identically zero (a single token has dQ = dK = 0)."""
     mask = ~np.isnan(want)
     assert np.isfinite(got[mask]).all(), f"{name}: non-finite values"
-    rel = brute.rel_max(got[mask], want[mask])
-    assert rel <= tol, f"{name}: relative error {rel:.3e} exceeds {tol}"
-    return rel
+    err = brute.max_abs(got[mask], want[mask])
+    scale = float(np.max(np.abs(want[mask])))
+    assert err <= tol * scale + floor, f"{name}: error {err:.3e} exceeds {tol} * {scale:.3e}"
+    return err / max(scale, 1e-30)
