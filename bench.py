@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path: causal flash-attention forward + backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config nstar|c1|c2|c3|c4|c5]
+
+A step is one forward + one backward pass of attention over one synthetic batch that is already resident
+in HBM.  The default workload is the target shape of the baseline (B=4, H=32, T=4096, d=128, bf16, causal);
+the five baseline configurations are timed briefly as well and reported under "configs".  One JSON line is
+printed.  FLOPs are the algorithmic ones of the baseline's work model: 2 (forward) + 5 (backward) matrix
+products of 2*T^2*d per (batch, query head), halved for the causal mask, i.e. 7*B*H*T^2*d in total;
+recomputation inside the two-kernel backward is not counted.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2516.6, "fp16": 2516.6, "fp32": 157.3}  # MI355X dense MFMA (256 CU x 2.4 GHz)
+
+# name: (B, Hq, Hkv, T, d, dtype, sigma_qk, description)
+CONFIGS = {
+    "c1": (4, 4, 4, 48, 16, "fp32", 1.0, "tiny quickstart LM attention B4 H4 T48 d16 fp32"),
+    "c2": (8, 12, 12, 1024, 64, "bf16", 0.70710678, "GPT-2-small-shaped B8 H12 T1024 d64 bf16"),
+    "c3": (4, 32, 32, 2048, 128, "bf16", 1.0, "Llama-7B-shaped B4 H32 T2048 d128 bf16"),
+    "c4": (4, 32, 8, 4096, 128, "bf16", 1.0, "GQA B4 Hq32/Hkv8 T4096 d128 bf16"),
+    "c5": (1, 16, 16, 16384, 64, "fp16", 3.0, "long-context B1 H16 T16384 d64 fp16"),
+    "nstar": (4, 32, 32, 4096, 128, "bf16", 1.0, "target shape B4 H32 T4096 d128 bf16 causal"),
+}
+SEEDS = {"c1": 1, "c2": 2, "c3": 3, "c4": 4, "c5": 5, "nstar": 6}
+# algorithmic matrix products per kernel (units of B*H*T^2*d FLOPs, causal-halved)
+KERNEL_UNITS = {"fwd_mfma": 2.0, "dkdv_mfma": 4.0, "dq_mfma": 1.0, "fwd_f32": 2.0, "dkdv_f32": 4.0, "dq_f32": 1.0}
+
+
+def make_inputs(torch, name):
+    b, hq, hkv, t, d, dtype, sigma, _ = CONFIGS[name]
+    tdt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[dtype]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5E17 + SEEDS[name])
+    q = (sigma * torch.randn(b, hq, t, d, device="cuda", generator=gen)).to(tdt)
+    k = (sigma * torch.randn(b, hkv, t, d, device="cuda", generator=gen)).to(tdt)
+    v = torch.randn(b, hkv, t, d, device="cuda", generator=gen).to(tdt)
+    g = torch.randn(b, hq, t, d, device="cuda", generator=gen).to(tdt)
+    return q, k, v, g
+
+
+class Workload:
+    def __init__(self, torch, name):
+        import sentinel_amd
+        self.torch = torch
+        self.fa = sentinel_amd
+        self.name = name
+        self.b, self.hq, self.hkv, self.t, self.d, self.dtype, _, self.desc = CONFIGS[name]
+        self.q, self.k, self.v, self.g = make_inputs(torch, name)
+        self.out = torch.empty_like(self.q)
+        self.lse = torch.empty(self.b, self.hq, self.t, dtype=torch.float32, device="cuda")
+        self.dq, self.dk, self.dv = torch.empty_like(self.q), torch.empty_like(self.k), torch.empty_like(self.v)
+        self.delta = torch.empty(self.hq, self.b * self.t, dtype=torch.float32, device="cuda")
+        self.unit_flops = float(self.b) * self.hq * self.t * self.t * self.d
+
+    def forward(self):
+        self.fa.flash_attention_forward(self.q, self.k, self.v, out=self.out, lse=self.lse)
+
+    def backward(self):
+        self.fa.flash_attention_backward(self.q, self.k, self.v, self.out, self.lse, self.g, dq=self.dq, dk=self.dk,
+                                         dv=self.dv, delta=self.delta)
+
+    def step(self):
+        self.forward()
+        self.backward()
+
+    def timed(self, fn, steps, warmup):
+        torch = self.torch
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3  # ms per call
+
+    def kernel_times(self, steps):
+        """Average duration of each kernel over `steps` timed steps (hipEvents on the launch stream)."""
+        self.fa.set_kernel_timing(True)
+        self.fa.collect_kernel_timings()
+        for _ in range(steps):
+            self.step()
+        times = self.fa.collect_kernel_timings()
+        self.fa.set_kernel_timing(False)
+        return {k: total / max(n, 1) for k, (total, n) in times.items()}
+
+
+def cpu_baseline(name, heads_sample):
+    """The CPU oracle (a restatement of the reference's OpenMP attention) timed on a bounded sample."""
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib
+    b, hq, hkv, t, d, dtype, sigma, _ = CONFIGS[name]
+    group = hq // hkv
+    heads_sample = max(group, min(hq, heads_sample) // group * group)
+    kv_sample = heads_sample // group
+    rng = np.random.default_rng(0x5E17)
+    q = (sigma * rng.standard_normal((heads_sample * d, t))).astype(np.float32)
+    k = (sigma * rng.standard_normal((kv_sample * d, t))).astype(np.float32)
+    v = rng.standard_normal((kv_sample * d, t)).astype(np.float32)
+    g = rng.standard_normal((heads_sample * d, t)).astype(np.float32)
+    threads = oracle_lib.oracle().sentinel_oracle_max_threads()
+    t0 = time.perf_counter()
+    oracle_lib.oracle_attention(q, k, v, g, q_heads=heads_sample, kv_heads=kv_sample, head_dim=d, seq_len=t)
+    dt = time.perf_counter() - t0
+    flops = 7.0 * heads_sample * t * t * d
+    return {
+        "value": flops / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"1 sequence x {heads_sample} of {b * hq} (batch, head) pairs of {name}, fp32, forward+backward, "
+                  f"{dt:.1f} s; gemm/softmax OpenMP-parallel as in the reference's single-call mode; "
+                  "same causal FLOP count although the CPU path multiplies the full T x T",
+        "seconds": dt,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="nstar", choices=sorted(CONFIGS))
+    ap.add_argument("--cpu-heads", type=int, default=8, help="(batch, head) pairs in the CPU baseline sample; 0 = skip")
+    ap.add_argument("--no-configs", action="store_true", help="skip the brief timing of the other configurations")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU only; attention shards over (batch, kv-head group) with no "
+              "exchange, so a multi-GPU figure would be N independent copies of this one", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import sentinel_amd
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    sentinel_amd.load_library()
+
+    w = Workload(torch, args.config)
+    ms_step = w.timed(w.step, args.steps, args.warmup)
+    ms_fwd = w.timed(w.forward, max(args.steps // 2, 1), 1)
+    ms_bwd = w.timed(w.backward, max(args.steps // 2, 1), 1)
+    kernels = w.kernel_times(args.steps)
+    total_flops = 7.0 * w.unit_flops
+    value = total_flops / (ms_step * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[w.dtype]
+
+    counted = {k: v for k, v in kernels.items() if k in KERNEL_UNITS}
+    dominant = max(counted, key=counted.get)
+    achieved = KERNEL_UNITS[dominant] * w.unit_flops / (counted[dominant] * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                "frac": achieved / peak, "traffic": None,
+                "kernel_ms": counted[dominant],
+                "algorithmic_flops_per_launch": KERNEL_UNITS[dominant] * w.unit_flops}
+
+    line = {
+        "metric": "causal flash-attn fwd+bwd TFLOP/s",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": w.dtype,
+        "data": "synthetic",
+        "config": {"workload": w.desc, "batch": w.b, "q_heads": w.hq, "kv_heads": w.hkv, "seq_len": w.t, "head_dim": w.d,
+                   "causal": True, "layout": "[B,H,T,d]"},
+        "pct_of_mfma_peak": 100.0 * value / peak,
+        "fwd_ms": ms_fwd,
+        "bwd_ms": ms_bwd,
+        "fwd_tflops": 2.0 * w.unit_flops / (ms_fwd * 1e-3) / 1e12,
+        "bwd_tflops": 5.0 * w.unit_flops / (ms_bwd * 1e-3) / 1e12,
+        "kernels_ms": kernels,
+        "roofline": roofline,
+    }
+
+    if not args.no_configs:
+        others = {}
+        for name in ("c1", "c2", "c3", "c4", "c5"):
+            if name == args.config:
+                continue
+            o = Workload(torch, name)
+            steps = 10 if name != "c1" else 50
+            f_ms = o.timed(o.forward, steps, 2)
+            b_ms = o.timed(o.backward, steps, 2)
+            tf = 7.0 * o.unit_flops / ((f_ms + b_ms) * 1e-3) / 1e12
+            others[name] = {"workload": o.desc, "dtype": o.dtype, "fwd_ms": f_ms, "bwd_ms": b_ms, "tflops": tf,
+                            "pct_of_mfma_peak": 100.0 * tf / PEAK_TFLOPS[o.dtype]}
+            del o
+            torch.cuda.empty_cache()
+        line["configs"] = others
+
+    if args.cpu_heads > 0:
+        line["cpu_baseline"] = cpu_baseline(args.config, args.cpu_heads)
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -112,6 +112,18 @@ SENTINEL_HIP_API const char* sentinel_hip_strerror(int code);
 /* Detail of the last non-OK return on the calling thread ("" if none). */
 SENTINEL_HIP_API const char* sentinel_hip_last_error(void);
 
+/*
+ * Optional per-kernel timing (diagnostics). Stands for the cudaEvent phase breakdown of
+ * CudaLanguageModel::runTrainProfileDemo (sentinel/NeuralNet/Cuda/CudaLanguageModel.cu:4203-4211, :4378).
+ * While enabled, every kernel launched by the entry points above is bracketed by two hipEvents on its
+ * stream (so such calls must not be captured into a graph). sentinel_hip_flash_collect_timings waits for
+ * the recorded events, adds the durations up per kernel name since the previous collect, writes at most
+ * `capacity` entries (names are static strings) and returns the number written.
+ */
+SENTINEL_HIP_API int sentinel_hip_flash_set_timing(int enabled); /* returns the previous setting */
+SENTINEL_HIP_API int sentinel_hip_flash_collect_timings(const char** names_out, float* total_ms_out, int* launches_out,
+                                                        int capacity);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,8 +1,10 @@
 """MI355X-native causal flash attention behind Sentinel's CudaFlashAttention interface."""
 from .flash_attention import (  # noqa: F401
     HipFlashAttention,
+    collect_kernel_timings,
     flash_attention_backward,
     flash_attention_forward,
     library_path,
     load_library,
+    set_kernel_timing,
 )

@@ -153,6 +153,14 @@ extern "C" const char* sentinel_hip_strerror(int code) {
 
 extern "C" const char* sentinel_hip_last_error(void) { return g_last_error; }
 
+extern "C" int sentinel_hip_flash_set_timing(int enabled) { return timing_set_enabled(enabled); }
+
+extern "C" int sentinel_hip_flash_collect_timings(const char** names_out, float* total_ms_out, int* launches_out,
+                                                  int capacity) {
+    if (!names_out || !total_ms_out || !launches_out || capacity <= 0) return 0;
+    return timing_collect(names_out, total_ms_out, launches_out, capacity);
+}
+
 extern "C" size_t sentinel_hip_flash_workspace_bytes(int io_dtype, int compute_dtype, int layout, int q_heads, int kv_heads,
                                                      int head_dim, int seq_len, int pack_count, int backward) {
     Resolved r;

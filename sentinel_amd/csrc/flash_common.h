@@ -61,5 +61,21 @@ hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int he
 hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,
                                   int seq_len, int packs, hipStream_t stream);
 
+// ---- optional per-kernel hipEvent timing (kernel_timing.hip) ----
+class KernelTimer {
+public:
+    KernelTimer(const char* name, hipStream_t stream);
+    ~KernelTimer();
+    KernelTimer(const KernelTimer&) = delete;
+    KernelTimer& operator=(const KernelTimer&) = delete;
+
+private:
+    const char* name_;
+    hipStream_t stream_;
+    hipEvent_t start_;
+};
+int timing_set_enabled(int enabled);
+int timing_collect(const char** names, float* total_ms, int* launches, int capacity);
+
 }  // namespace sentinel_hip
 #endif

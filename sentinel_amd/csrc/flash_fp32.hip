@@ -314,6 +314,7 @@ template <int DP>
 hipError_t run_fwd(const float* q, const float* k, const float* v, float* out, float* lse, TensorMap qm, TensorMap kvm,
                    RowMap lm, AttnGeom g, hipStream_t stream) {
     const dim3 grid((g.seq_len + kLanes - 1) / kLanes, g.q_heads, g.packs);
+    KernelTimer timer("fwd_f32", stream);
     hipLaunchKernelGGL(fwd_f32_kernel<DP>, grid, dim3(kLanes), 0, stream, q, k, v, out, lse, qm, kvm, lm, g);
     return hipGetLastError();
 }
@@ -323,9 +324,13 @@ hipError_t run_bwd(const float* q, const float* k, const float* v, const float* 
                    const float* delta, float* dq, float* dk, float* dv, TensorMap qm, TensorMap kvm, RowMap lm, AttnGeom g,
                    hipStream_t stream) {
     const int tiles = (g.seq_len + kLanes - 1) / kLanes;
-    hipLaunchKernelGGL(bwd_dq_f32_kernel<DP>, dim3(tiles, g.q_heads, g.packs), dim3(kLanes), 0, stream, q, k, v, lse, d_out,
-                       delta, dq, qm, kvm, lm, g);
-    hipError_t err = hipGetLastError();
+    hipError_t err;
+    {
+        KernelTimer timer("dq_f32", stream);
+        hipLaunchKernelGGL(bwd_dq_f32_kernel<DP>, dim3(tiles, g.q_heads, g.packs), dim3(kLanes), 0, stream, q, k, v, lse,
+                           d_out, delta, dq, qm, kvm, lm, g);
+        err = hipGetLastError();
+    }
     if (err != hipSuccess) return err;
 
     const size_t lds = dkdv_lds_bytes<DP>();
@@ -336,6 +341,7 @@ hipError_t run_bwd(const float* q, const float* k, const float* v, const float* 
         if (err != hipSuccess) return err;
         raised = true;
     }
+    KernelTimer timer("dkdv_f32", stream);
     hipLaunchKernelGGL(bwd_dkdv_f32_kernel<DP>, dim3(tiles, g.kv_heads, g.packs), dim3(kLanes), lds, stream, q, k, v, lse,
                        d_out, delta, dk, dv, qm, kvm, lm, g);
     return hipGetLastError();
@@ -354,9 +360,13 @@ hipError_t launch_fwd_f32(const float* q, const float* k, const float* v, float*
 hipError_t launch_bwd_f32(const float* q, const float* k, const float* v, const float* out, const float* lse,
                           const float* d_out, float* dq, float* dk, float* dv, float* delta, TensorMap qm, TensorMap kvm,
                           RowMap lm, AttnGeom g, hipStream_t stream) {
-    hipLaunchKernelGGL(delta_f32_kernel, dim3((g.seq_len + 127) / 128, g.q_heads, g.packs), dim3(128), 0, stream, out,
-                       d_out, delta, qm, g);
-    hipError_t err = hipGetLastError();
+    hipError_t err;
+    {
+        KernelTimer timer("delta_f32", stream);
+        hipLaunchKernelGGL(delta_f32_kernel, dim3((g.seq_len + 127) / 128, g.q_heads, g.packs), dim3(128), 0, stream, out,
+                           d_out, delta, qm, g);
+        err = hipGetLastError();
+    }
     if (err != hipSuccess) return err;
     if (g.head_dim <= 16) return run_bwd<16>(q, k, v, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);
     if (g.head_dim <= 32) return run_bwd<32>(q, k, v, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);

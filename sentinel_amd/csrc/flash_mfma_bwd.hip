@@ -457,9 +457,13 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
     const int T = g.seq_len;
 
     constexpr int RPB = kBwdThreads / (D / 8);
-    hipLaunchKernelGGL((delta_mfma_kernel<E, D>), dim3((T + RPB - 1) / RPB, g.q_heads, g.packs), dim3(kBwdThreads), 0,
-                       stream, op, gp, delta, g);
-    hipError_t err = hipGetLastError();
+    hipError_t err;
+    {
+        KernelTimer timer("delta_mfma", stream);
+        hipLaunchKernelGGL((delta_mfma_kernel<E, D>), dim3((T + RPB - 1) / RPB, g.q_heads, g.packs), dim3(kBwdThreads), 0,
+                           stream, op, gp, delta, g);
+        err = hipGetLastError();
+    }
     if (err != hipSuccess) return err;
 
     // dK, dV
@@ -477,6 +481,7 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
             if (err != hipSuccess) return err;
             raised[which] = true;
         }
+        KernelTimer timer("dkdv_mfma", stream);
         if (g.causal)
             hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, true>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp,
                                lse, delta, dkp, dvp, lm, g, k_tiles, total);
@@ -491,6 +496,7 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
         const int q_tiles = (T + kDqQueryTile - 1) / kDqQueryTile;
         const int total = g.packs * g.q_heads * q_tiles;
         const int grid = (total + 7) / 8 * 8;
+        KernelTimer timer("dq_mfma", stream);
         if (g.causal)
             hipLaunchKernelGGL((dq_mfma_kernel<E, D, true>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp, lse,
                                delta, dqp, lm, g, q_tiles, total);

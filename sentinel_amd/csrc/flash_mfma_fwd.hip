@@ -209,6 +209,7 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
     auto kp = static_cast<const unsigned short*>(k);
     auto vp = static_cast<const unsigned short*>(v);
     auto op = static_cast<unsigned short*>(out);
+    KernelTimer timer("fwd_mfma", stream);
     if (g.causal)
         hipLaunchKernelGGL((fwd_mfma_kernel<E, D, true>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm,
                            g, q_tiles, total);

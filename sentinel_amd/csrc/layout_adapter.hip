@@ -73,6 +73,7 @@ hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int he
                                   int seq_len, int packs, hipStream_t stream) {
     const dim3 grid((seq_len + kTile - 1) / kTile, (head_dim + kTile - 1) / kTile, packs * heads);
     auto out = static_cast<unsigned short*>(dst);
+    KernelTimer timer("columns_to_bhtd", stream);
     if (type == Elem::BF16)
         hipLaunchKernelGGL(columns_to_bhtd_kernel<Bf16>, grid, dim3(256), 0, stream, src, out, heads, head_dim,
                            (long long)stride_columns, seq_len);
@@ -88,6 +89,7 @@ hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int he
                                   int seq_len, int packs, hipStream_t stream) {
     const dim3 grid((seq_len + kTile - 1) / kTile, (head_dim + kTile - 1) / kTile, packs * heads);
     auto in = static_cast<const unsigned short*>(src);
+    KernelTimer timer("bhtd_to_columns", stream);
     if (type == Elem::BF16)
         hipLaunchKernelGGL(bhtd_to_columns_kernel<Bf16>, grid, dim3(256), 0, stream, in, dst, heads, head_dim,
                            (long long)stride_columns, seq_len);

@@ -57,8 +57,28 @@ def load_library():
     lib.sentinel_hip_strerror.argtypes = [i]
     lib.sentinel_hip_strerror.restype = ctypes.c_char_p
     lib.sentinel_hip_last_error.restype = ctypes.c_char_p
+    lib.sentinel_hip_flash_set_timing.argtypes = [i]
+    lib.sentinel_hip_flash_set_timing.restype = i
+    lib.sentinel_hip_flash_collect_timings.argtypes = [ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(f),
+                                                       ctypes.POINTER(i), i]
+    lib.sentinel_hip_flash_collect_timings.restype = i
     _lib = lib
     return lib
+
+
+def set_kernel_timing(enabled):
+    """Bracket every kernel launch with hipEvents (diagnostics; not for captured graphs). Returns the old setting."""
+    return bool(load_library().sentinel_hip_flash_set_timing(int(bool(enabled))))
+
+
+def collect_kernel_timings(capacity=32):
+    """{kernel name: (total milliseconds, launches)} since the previous collect; waits for the recorded events."""
+    lib = load_library()
+    names = (ctypes.c_char_p * capacity)()
+    total = (ctypes.c_float * capacity)()
+    launches = (ctypes.c_int * capacity)()
+    count = lib.sentinel_hip_flash_collect_timings(names, total, launches, capacity)
+    return {names[j].decode(): (float(total[j]), int(launches[j])) for j in range(count)}
 
 
 def _check(code):
