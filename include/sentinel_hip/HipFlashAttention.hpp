@@ -1,0 +1,225 @@
+// Header-only C++ face of the HIP attention library for Sentinel's host code.
+//
+// HipMatrix mirrors the parts of CudaMatrix the attention dispatch touches
+// (sentinel/NeuralNet/Cuda/CudaMatmul.hpp:100-171: rows, cols, buffer.deviceData, ensureSize, upload,
+// download) and HipFlashAttention mirrors class CudaFlashAttention
+// (sentinel/NeuralNet/Cuda/CudaFlashAttention.hpp:12-41): same static methods, argument order, defaults,
+// output resizing (CudaFlashAttention.cu:1555-1556, :1633-1640) and exception types
+// (std::invalid_argument for shape / window errors, std::runtime_error for device errors).
+// Extra trailing argument kvHeadCount (0 = same as headCount) exposes native grouped-query attention.
+// Link against libsentinel_hip_attn.so and the HIP runtime.
+#ifndef SENTINEL_HIP_HIPFLASHATTENTION_HPP
+#define SENTINEL_HIP_HIPFLASHATTENTION_HPP
+
+#include "../sentinel_hip_attn.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace sentinel_hip_host {
+
+inline void throwIfHipFailed(hipError_t status, const char* what) {
+    if (status != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(status));
+}
+
+/// reusable device float buffer, grows only when capacity is too small
+class HipDeviceBuffer {
+public:
+    float* deviceData = nullptr;
+    size_t capacityBytes = 0;
+
+    HipDeviceBuffer() = default;
+    ~HipDeviceBuffer() { this->free(); }
+    HipDeviceBuffer(const HipDeviceBuffer&) = delete;
+    HipDeviceBuffer& operator=(const HipDeviceBuffer&) = delete;
+    HipDeviceBuffer(HipDeviceBuffer&& other) noexcept : deviceData(other.deviceData), capacityBytes(other.capacityBytes) {
+        other.deviceData = nullptr;
+        other.capacityBytes = 0;
+    }
+    HipDeviceBuffer& operator=(HipDeviceBuffer&& other) noexcept {
+        if (this != &other) {
+            this->free();
+            deviceData = other.deviceData;
+            capacityBytes = other.capacityBytes;
+            other.deviceData = nullptr;
+            other.capacityBytes = 0;
+        }
+        return *this;
+    }
+    void ensureCapacity(size_t requiredBytes) {
+        if (requiredBytes <= capacityBytes) return;
+        this->free();
+        throwIfHipFailed(hipMalloc(reinterpret_cast<void**>(&deviceData), requiredBytes), "HipDeviceBuffer hipMalloc");
+        capacityBytes = requiredBytes;
+    }
+    void free() {
+        if (deviceData) (void)hipFree(deviceData);
+        deviceData = nullptr;
+        capacityBytes = 0;
+    }
+};
+
+/// row major float matrix that lives on the device
+class HipMatrix {
+public:
+    size_t rows = 0;
+    size_t cols = 0;
+    HipDeviceBuffer buffer;
+
+    HipMatrix() = default;
+    HipMatrix(HipMatrix&&) noexcept = default;
+    HipMatrix& operator=(HipMatrix&&) noexcept = default;
+
+    bool empty() const { return rows == 0 || cols == 0; }
+    size_t elementCount() const { return rows * cols; }
+    size_t byteCount() const { return rows * cols * sizeof(float); }
+    void ensureSize(size_t rowCount, size_t columnCount) {
+        rows = rowCount;
+        cols = columnCount;
+        buffer.ensureCapacity(byteCount());
+    }
+    void upload(const std::vector<float>& host, size_t rowCount, size_t columnCount) {
+        if (host.size() != rowCount * columnCount) throw std::invalid_argument("HipMatrix::upload size mismatch");
+        ensureSize(rowCount, columnCount);
+        throwIfHipFailed(hipMemcpy(buffer.deviceData, host.data(), byteCount(), hipMemcpyHostToDevice), "HipMatrix::upload");
+    }
+    std::vector<float> download() const {
+        std::vector<float> host(elementCount());
+        throwIfHipFailed(hipDeviceSynchronize(), "HipMatrix::download sync");
+        throwIfHipFailed(hipMemcpy(host.data(), buffer.deviceData, byteCount(), hipMemcpyDeviceToHost), "HipMatrix::download");
+        return host;
+    }
+    void fill(float value) { upload(std::vector<float>(elementCount(), value), rows, cols); }
+};
+
+class HipFlashAttention {
+public:
+    static constexpr int queryTileSize = 128;
+    static constexpr int keyTileSize = 64;
+    static constexpr int maxHeadDimension = 128;
+
+    /// arithmetic for the matrix products: SENTINEL_HIP_COMPUTE_AUTO (exact fp32 for these fp32 matrices),
+    /// SENTINEL_HIP_COMPUTE_BF16 or SENTINEL_HIP_COMPUTE_F16 (MFMA, head_dim 64 / 128)
+    static int& computeType() {
+        static int value = SENTINEL_HIP_COMPUTE_AUTO;
+        return value;
+    }
+
+    /// process-wide launch stream (stands for CudaMatmul::activeStream, CudaMatmul.cu:493-506)
+    static hipStream_t& activeStream() {
+        static hipStream_t stream = nullptr;
+        return stream;
+    }
+
+    static void forward(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, HipMatrix& out,
+                        HipMatrix& logSumExp, float scale, bool causal = true) {
+        forwardMultiHead(query, key, value, out, logSumExp, 1, static_cast<int>(query.rows), scale, causal, 0,
+                         static_cast<int>(query.cols));
+    }
+
+    static void forwardMultiHead(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, HipMatrix& out,
+                                 HipMatrix& logSumExp, int headCount, int headDimension, float scale, bool causal = true,
+                                 int columnStart = 0, int columnCount = 0, int packCount = 1, int kvHeadCount = 0) {
+        const char* op = "HipFlashAttention::forwardMultiHead";
+        const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
+        if (!sentinel_hip_device_available()) throw std::runtime_error(std::string(op) + " no HIP device");
+        out.ensureSize(query.rows, query.cols);
+        logSumExp.ensureSize(static_cast<size_t>(headCount), query.cols);
+        void* ws = nullptr;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws);
+        check(sentinel_hip_flash_fwd(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
+                                     out.buffer.deviceData, logSumExp.buffer.deviceData, SENTINEL_HIP_F32, computeType(),
+                                     SENTINEL_HIP_LAYOUT_COLUMNS, headCount, kvHeads, headDimension,
+                                     static_cast<int>(query.cols), columnStart, columnCount, packCount, scale, causal ? 1 : 0,
+                                     ws, wsBytes, activeStream()));
+    }
+
+    static void backward(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, const HipMatrix& out,
+                         const HipMatrix& logSumExp, const HipMatrix& outGradient, HipMatrix& queryGradient,
+                         HipMatrix& keyGradient, HipMatrix& valueGradient, float scale, bool causal = true) {
+        HipMatrix deltaWorkspace;
+        backwardMultiHead(query, key, value, out, logSumExp, outGradient, queryGradient, keyGradient, valueGradient,
+                          deltaWorkspace, 1, static_cast<int>(query.rows), scale, causal, 0, static_cast<int>(query.cols));
+        throwIfHipFailed(hipStreamSynchronize(activeStream()), "HipFlashAttention::backward");  // deltaWorkspace dies here
+    }
+
+    static void backwardMultiHead(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, const HipMatrix& out,
+                                  const HipMatrix& logSumExp, const HipMatrix& outGradient, HipMatrix& queryGradient,
+                                  HipMatrix& keyGradient, HipMatrix& valueGradient, HipMatrix& deltaWorkspace, int headCount,
+                                  int headDimension, float scale, bool causal = true, int columnStart = 0,
+                                  int columnCount = 0, int packCount = 1, int kvHeadCount = 0) {
+        const char* op = "HipFlashAttention::backwardMultiHead";
+        const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
+        if (out.rows != query.rows || out.cols != query.cols) throw std::invalid_argument(std::string(op) + " out shape mismatch");
+        if (outGradient.rows != query.rows || outGradient.cols != query.cols)
+            throw std::invalid_argument(std::string(op) + " outGradient shape mismatch");
+        if (logSumExp.rows != static_cast<size_t>(headCount) || logSumExp.cols != query.cols)
+            throw std::invalid_argument(std::string(op) + " logSumExp shape mismatch");
+        if (!sentinel_hip_device_available()) throw std::runtime_error(std::string(op) + " no HIP device");
+        if (packCount <= 0) packCount = 1;
+        int resolvedCount = columnCount > 0 ? columnCount : static_cast<int>(query.cols) - columnStart;
+        if (columnStart < 0 || resolvedCount <= 0 || columnStart + resolvedCount > static_cast<int>(query.cols))
+            throw std::invalid_argument("HipFlashAttention invalid column window");
+        queryGradient.ensureSize(query.rows, query.cols);
+        keyGradient.ensureSize(key.rows, key.cols);
+        valueGradient.ensureSize(value.rows, value.cols);
+        deltaWorkspace.ensureSize(static_cast<size_t>(headCount), static_cast<size_t>(packCount) * static_cast<size_t>(resolvedCount));
+        void* ws = nullptr;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws);
+        check(sentinel_hip_flash_bwd(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
+                                     out.buffer.deviceData, logSumExp.buffer.deviceData, outGradient.buffer.deviceData,
+                                     queryGradient.buffer.deviceData, keyGradient.buffer.deviceData,
+                                     valueGradient.buffer.deviceData, deltaWorkspace.buffer.deviceData, SENTINEL_HIP_F32,
+                                     computeType(), SENTINEL_HIP_LAYOUT_COLUMNS, headCount, kvHeads, headDimension,
+                                     static_cast<int>(query.cols), columnStart, columnCount, packCount, scale, causal ? 1 : 0,
+                                     ws, wsBytes, activeStream()));
+    }
+
+private:
+    // validateMultiHeadShape (CudaFlashAttention.cu:1458-1471), K/V rows rule widened to grouped heads
+    static int validateMultiHeadShape(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, int headCount,
+                                      int headDimension, int kvHeadCount, const char* op) {
+        const std::string name(op);
+        if (query.empty() || key.empty() || value.empty()) throw std::invalid_argument(name + " empty input");
+        if (headCount <= 0 || headDimension <= 0) throw std::invalid_argument(name + " invalid head geometry");
+        if (headDimension > maxHeadDimension) throw std::invalid_argument(name + " headDim exceeds maxHeadDimension");
+        const int kvHeads = kvHeadCount <= 0 ? headCount : kvHeadCount;
+        if (headCount % kvHeads != 0) throw std::invalid_argument(name + " headCount must be divisible by kvHeadCount");
+        if (query.rows != static_cast<size_t>(headCount) * static_cast<size_t>(headDimension))
+            throw std::invalid_argument(name + " query rows mismatch headCount*headDim");
+        if (key.rows != static_cast<size_t>(kvHeads) * static_cast<size_t>(headDimension) || value.rows != key.rows)
+            throw std::invalid_argument(name + " key/value rows mismatch");
+        if (query.cols != key.cols || query.cols != value.cols) throw std::invalid_argument(name + " sequenceLength mismatch");
+        return kvHeads;
+    }
+
+    // Scratch for MFMA arithmetic on Sentinel's layout; one process-wide buffer that only grows (its first
+    // growth allocates, so warm it up before capturing a graph).
+    static size_t workspaceFor(int headCount, int kvHeads, int headDimension, const HipMatrix& query, int columnStart,
+                               int columnCount, int packCount, bool backward, void*& ws) {
+        static HipDeviceBuffer scratch;
+        const int resolved = columnCount > 0 ? columnCount : static_cast<int>(query.cols) - columnStart;
+        const size_t need = sentinel_hip_flash_workspace_bytes(SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS,
+                                                               headCount, kvHeads, headDimension, resolved > 0 ? resolved : 1,
+                                                               packCount > 0 ? packCount : 1, backward ? 1 : 0);
+        if (need == 0) return 0;
+        scratch.ensureCapacity(need);
+        ws = scratch.deviceData;
+        return need;
+    }
+
+    static void check(int code) {
+        if (code == SENTINEL_HIP_OK) return;
+        std::string detail = sentinel_hip_last_error();
+        if (detail.empty()) detail = sentinel_hip_strerror(code);
+        if (code == SENTINEL_HIP_RUNTIME) throw std::runtime_error(detail);
+        throw std::invalid_argument(detail);
+    }
+};
+
+}  // namespace sentinel_hip_host
+#endif

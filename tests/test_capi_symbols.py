@@ -1,0 +1,75 @@
+"""CPU-only checks of the boundary: the built library exports every symbol the header declares, argument
+validation returns the documented codes without touching a GPU, and the Python mirror refuses to run without it."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "sentinel_hip_attn.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    return sorted(set(re.findall(r"SENTINEL_HIP_API\s+[\w\s\*]+?\b(sentinel_hip_\w+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import sentinel_amd
+    if not os.path.exists(sentinel_amd.library_path()):
+        from sentinel_amd.build import build_library
+        build_library()
+    return sentinel_amd.load_library()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = _declared()
+    assert len(names) >= 9, names
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+
+
+def test_codes_and_messages_without_a_gpu(lib):
+    assert lib.sentinel_hip_flash_max_head_dim() == 128
+    assert lib.sentinel_hip_strerror(0) == b"ok"
+    fwd = lib.sentinel_hip_flash_fwd
+    one = ctypes.c_void_p(16)  # never dereferenced: validation fails first
+
+    def call(**kw):
+        a = dict(io=0, comp=-1, layout=0, hq=4, hkv=4, d=16, stride=192, col0=0, t=48, packs=4, scale=0.25)
+        a.update(kw)
+        return fwd(one, one, one, one, one, a["io"], a["comp"], a["layout"], a["hq"], a["hkv"], a["d"], a["stride"], a["col0"],
+                   a["t"], a["packs"], a["scale"], 1, None, 0, None)
+
+    assert fwd(None, one, one, one, one, 0, -1, 0, 4, 4, 16, 192, 0, 48, 4, 0.25, 1, None, 0, None) == 1
+    assert b"empty input" in lib.sentinel_hip_last_error()
+    assert call(hq=0) == 1 and b"invalid head geometry" in lib.sentinel_hip_last_error()
+    assert call(hq=3, hkv=2) == 1 and b"divisible by kvHeadCount" in lib.sentinel_hip_last_error()
+    assert call(d=256) == 1 and b"headDim exceeds maxHeadDimension" in lib.sentinel_hip_last_error()
+    assert call(col0=190) == 1 and b"invalid column window" in lib.sentinel_hip_last_error()
+    assert call(packs=5) == 1 and b"pack window exceeds columns" in lib.sentinel_hip_last_error()
+    assert call(scale=0.0) == 1 and b"scale must be positive" in lib.sentinel_hip_last_error()
+    assert call(comp=1) == 2 and b"head_dim 64 and 128" in lib.sentinel_hip_last_error()   # d=16 has no MFMA kernel
+    assert call(io=1, layout=0, d=64) == 2                                        # 16-bit needs [B,H,T,d]
+    # a valid call without a device is a runtime error, not a silent fallback
+    if not lib.sentinel_hip_device_available():
+        assert call() == 3 and b"no HIP device" in lib.sentinel_hip_last_error()
+
+
+def test_workspace_sizes(lib):
+    ws = lib.sentinel_hip_flash_workspace_bytes
+    assert ws(0, -1, 0, 4, 4, 16, 48, 4, 1) == 0          # fp32 arithmetic needs none
+    assert ws(1, -1, 1, 32, 8, 128, 4096, 4, 1) == 0      # native 16-bit layout needs none
+    nq, nkv = 4 * 32 * 4096 * 128 * 2, 4 * 8 * 4096 * 128 * 2
+    assert ws(0, 1, 0, 32, 8, 128, 4096, 4, 0) == 2 * nq + 2 * nkv
+    assert ws(0, 1, 0, 32, 8, 128, 4096, 4, 1) == 4 * nq + 4 * nkv
+
+
+def test_python_mirror_has_no_fallback(monkeypatch):
+    import sentinel_amd.flash_attention as fa
+    monkeypatch.setattr(fa, "_lib", None)
+    monkeypatch.setattr(fa, "_LIB_PATH", "/nonexistent/libsentinel_hip_attn.so")
+    with pytest.raises(ImportError, match="no fallback"):
+        fa.load_library()

@@ -1,0 +1,64 @@
+"""The drop-in faces of the library on the GPU: the C++ shim (HipFlashAttention.hpp) and MFMA arithmetic on
+Sentinel's own fp32 column layout (the adapter path), both through the C ABI."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_util
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def test_cpp_shim_parity_and_exceptions():
+    exe = os.path.join(HERE, "cpp", "test_shim")
+    assert os.path.exists(exe), "tests/cpp/test_shim is not built: python -c 'import __graft_entry__ as g; g.build()'"
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=110)
+    print(proc.stdout, proc.stderr, flush=True)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "shim ok" in proc.stdout
+
+
+@pytest.mark.parametrize("compute", ["bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(12, 12, 64, 128, 1, 0, 0), (8, 2, 128, 200, 2, 4, 4), (2, 2, 64, 70, 3, 3, 1)])
+def test_columns_layout_with_mfma_arithmetic(compute, shape):
+    from sentinel_amd import HipFlashAttention
+    hq, hkv, d, t, packs, col0, pad = shape
+    print(f"case {compute} {shape}", flush=True)
+    q, k, v, g = gpu_util.make_inputs(hq, hkv, d, t, packs, seed=sum(shape), dtype=compute, col0=col0, pad=pad)
+    want = gpu_util.oracle(q, k, v, g, hq, hkv, d, t, packs, col0=col0)
+    qd, kd, vd, gd = (torch.from_numpy(x).cuda() for x in (q, k, v, g))
+    sentinel = 777.0
+    out = torch.full_like(qd, sentinel)
+    lse = torch.full((hq, q.shape[1]), sentinel, device="cuda")
+    scale = 1.0 / np.sqrt(np.float32(d))
+    out, lse = HipFlashAttention.forward_multi_head(qd, kd, vd, out, lse, hq, d, scale, True, col0, t, packs,
+                                                    kv_head_count=hkv, compute=compute)
+    dq, dk, dv = (torch.full_like(x, sentinel) for x in (qd, kd, vd))
+    dq, dk, dv, _ = HipFlashAttention.backward_multi_head(qd, kd, vd, out, lse, gd, dq, dk, dv, None, hq, d, scale, True,
+                                                          col0, t, packs, kv_head_count=hkv, compute=compute)
+    torch.cuda.synchronize()
+    for key, got in (("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
+        got = got.cpu().numpy()
+        outside = np.isnan(want[key])
+        assert np.all(got[outside] == sentinel), f"{key}: wrote outside the pack window"
+        # the backward consumes `out` rounded to 16 bit a second time (fp32 -> 16 bit adapter), still within the bar
+        gpu_util.assert_close_lowp(np.where(outside, np.nan, got), want[key], key)
+    got = lse.cpu().numpy()
+    outside = np.isnan(want["lse"])
+    assert np.all(got[outside] == sentinel)
+    gpu_util.assert_close_fp32(np.where(outside, np.nan, got), want["lse"], "lse", tol=1e-3)
+
+
+def test_unsupported_head_dim_is_reported_not_faked():
+    from sentinel_amd import HipFlashAttention
+    q = torch.zeros((4 * 48, 64), device="cuda")
+    with pytest.raises(ValueError, match="MFMA kernels cover head_dim 64 and 128"):
+        HipFlashAttention.forward_multi_head(q, q, q, None, None, 4, 48, 0.1, compute="bf16")
+    # the exact fp32 kernels take any head_dim <= 128
+    out, lse = HipFlashAttention.forward_multi_head(q + 0.01, q, q, None, None, 4, 48, 0.1)
+    assert torch.isfinite(out).all()
