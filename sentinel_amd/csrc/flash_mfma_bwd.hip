@@ -12,6 +12,8 @@
 //                       registers, replacing reduceKvHeadGradsInto, CudaCausalSelfAttention.cu:36-44);
 //   dq_mfma_kernel      query-outer: a workgroup owns 128 queries, keeps Q, dO (as B operands) and dQ^T in
 //                       registers and streams K / V tiles through LDS (recomputing S and dP).
+// Tiles sit row-major in LDS; the products that contract over tokens (dV, dK, dQ) read their A operand out
+// of the same tiles with transposing LDS reads, so nothing is staged twice.
 // In both kernels the score-like tiles are produced so that one lane owns one key (dK/dV kernel) or one
 // query (dQ kernel) and their registers are, after type conversion, directly the B operand of the
 // following product (see mfma_tile.h).
@@ -58,7 +60,7 @@ constexpr int kDqQueryTile = 128;
 constexpr int kDqKeyTile = 64;
 
 template <typename E, int D, bool CAUSAL>
-__global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dq_mfma_kernel(const unsigned short* __restrict__ q,
+__global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned short* __restrict__ q,
                                                                   const unsigned short* __restrict__ k,
                                                                   const unsigned short* __restrict__ v,
                                                                   const unsigned short* __restrict__ d_out,
@@ -67,16 +69,13 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dq_mfma_kernel
                                                                   unsigned short* __restrict__ dq, RowMap lm, AttnGeom g,
                                                                   int q_tiles, int total_tiles) {
     constexpr int KT = kDqKeyTile;
-    typedef RowTile<KT, D, kBwdThreads> RTile;
-    typedef TransposedTile<KT, D, kBwdThreads> TTile;
+    typedef RowTile<KT, D, kBwdThreads, 8> RTile;
     constexpr int KS = RTile::kStride;
-    constexpr int TS = TTile::kStride;
     constexpr int KSTEPS = D / 16;
     constexpr int CB = D / 32;
 
-    __shared__ __attribute__((aligned(16))) unsigned short k_lds[KT * KS];
-    __shared__ __attribute__((aligned(16))) unsigned short v_lds[KT * KS];
-    __shared__ __attribute__((aligned(16))) unsigned short kt_lds[D * TS];
+    __shared__ __attribute__((aligned(16))) unsigned short k_lds[2][KT * KS];
+    __shared__ __attribute__((aligned(16))) unsigned short v_lds[2][KT * KS];
 
     const int per_xcd = (int)gridDim.x / 8;
     const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
@@ -116,15 +115,16 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dq_mfma_kernel
     const int q_hi = min(T, (qt + 1) * kDqQueryTile);
     const int kv_tiles = CAUSAL ? (q_hi + KT - 1) / KT : (T + KT - 1) / KT;
 
+    const __amdgpu_buffer_rsrc_t k_rsrc = make_head_rsrc(kb, (long long)T * D * 2);
+    const __amdgpu_buffer_rsrc_t v_rsrc = make_head_rsrc(vb, (long long)T * D * 2);
+    const int ld_off = RTile::global_offset(tid);
+    const int st_off = RTile::lds_offset(tid);
     RTile ktile;
     RTile vtile;
-    TTile kttile;
-    ktile.load(kb, 0, T, tid);
-    vtile.load(vb, 0, T, tid);
-    kttile.load(kb, 0, T, tid);
-    ktile.store(k_lds, tid);
-    vtile.store(v_lds, tid);
-    kttile.store(kt_lds, tid);
+    ktile.load(k_rsrc, ld_off, 0);
+    vtile.load(v_rsrc, ld_off, 0);
+    ktile.store(k_lds[0], st_off);
+    vtile.store(v_lds[0], st_off);
     __syncthreads();
 
     f32x16 acc[CB];
@@ -134,39 +134,37 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dq_mfma_kernel
         for (int i = 0; i < 16; ++i) acc[cb][i] = 0.0f;
 
     const int k_off = row_perm(n) * KS + gh * 8;
-    const int t_off = n * TS + gh * 8;
+    const int t_off = transposed_read_offset(lane, KS);
 
     for (int j = 0; j < kv_tiles; ++j) {
+        const int buf = j & 1;
         const bool more = j + 1 < kv_tiles;
         if (more) {
-            ktile.load(kb, (j + 1) * KT, T, tid);
-            vtile.load(vb, (j + 1) * KT, T, tid);
-            kttile.load(kb, (j + 1) * KT, T, tid);
+            ktile.load(k_rsrc, ld_off, (j + 1) * KT * D * 2);
+            vtile.load(v_rsrc, ld_off, (j + 1) * KT * D * 2);
         }
         const int key0 = j * KT;
         const bool skip = CAUSAL && key0 > q0w + 31;
         if (!skip) {
-            f32x16 s[2];
-            f32x16 dp[2];
+            const bool need_mask = CAUSAL ? (key0 + KT - 1 > q0w) : (key0 + KT > T);
+            // two 32-key halves one after the other keeps the live score registers to one half
 #pragma unroll
             for (int kbk = 0; kbk < 2; ++kbk) {
+                f32x16 s;
+                f32x16 dp;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    s[kbk][i] = 0.0f;
-                    dp[kbk][i] = 0.0f;
+                    s[i] = 0.0f;
+                    dp[i] = 0.0f;
                 }
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) {
-                    const u32x4 ak = lds_read128(&k_lds[kbk * 32 * KS + k_off + ks * 16]);
-                    s[kbk] = E::mfma(ak, qf[ks], s[kbk]);
-                    const u32x4 av = lds_read128(&v_lds[kbk * 32 * KS + k_off + ks * 16]);
-                    dp[kbk] = E::mfma(av, gf[ks], dp[kbk]);
+                    const u32x4 ak = lds_read128(&k_lds[buf][kbk * 32 * KS + k_off + ks * 16]);
+                    s = E::mfma(ak, qf[ks], s);
+                    const u32x4 av = lds_read128(&v_lds[buf][kbk * 32 * KS + k_off + ks * 16]);
+                    dp = E::mfma(av, gf[ks], dp);
                 }
-            }
-            const bool need_mask = CAUSAL ? (key0 + KT - 1 > q0w) : (key0 + KT > T);
-            u32x4 dsf[4];
-#pragma unroll
-            for (int kbk = 0; kbk < 2; ++kbk) {
+                u32x4 dsf[2];
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -175,32 +173,30 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dq_mfma_kernel
 #pragma unroll
                         for (int w = 0; w < 2; ++w) {
                             const int i = half * 8 + 2 * e + w;
-                            float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kbk][i], c2, -lse2));
+                            float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -lse2));
                             if (need_mask) {
                                 const int key = key0 + kbk * 32 + perm_row_of_reg(i, gh);
                                 const bool dead = CAUSAL ? key > qrow : key >= T;
                                 if (dead) p = 0.0f;
                             }
-                            ds2[w] = p * (dp[kbk][i] - dl);
+                            ds2[w] = p * (dp[i] - dl);
                         }
-                        dsf[kbk * 2 + half][e] = E::pack2(ds2[0], ds2[1]);
+                        dsf[half][e] = E::pack2(ds2[0], ds2[1]);
+                    }
+                }
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) {
+                        const u32x4 a = lds_read_transposed(&k_lds[buf][t_off + (kbk * 32 + half * 16) * KS + cb * 32], KS);
+                        acc[cb] = E::mfma(a, dsf[half], acc[cb]);
                     }
                 }
             }
-#pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4) {
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    const u32x4 a = lds_read128(&kt_lds[cb * 32 * TS + t_off + c4 * 16]);
-                    acc[cb] = E::mfma(a, dsf[c4], acc[cb]);
-                }
-            }
         }
-        __syncthreads();
         if (more) {
-            ktile.store(k_lds, tid);
-            vtile.store(v_lds, tid);
-            kttile.store(kt_lds, tid);
+            ktile.store(k_lds[buf ^ 1], st_off);
+            vtile.store(v_lds[buf ^ 1], st_off);
         }
         __syncthreads();
     }
@@ -229,11 +225,8 @@ template <int D>
 struct DkvLds {
     static constexpr int QT = kDkvQueryTile;
     static constexpr int QS = D + 8;
-    static constexpr int TS = QT + 8;
     unsigned short q[QT * QS];
     unsigned short g[QT * QS];
-    unsigned short qt[D * TS];
-    unsigned short gt[D * TS];
     float lse2[QT];
     float dl[QT];
 };
@@ -245,11 +238,9 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
     int total_tiles) {
     constexpr int QT = kDkvQueryTile;
-    typedef RowTile<QT, D, kBwdThreads> RTile;
-    typedef TransposedTile<QT, D, kBwdThreads> TTile;
+    typedef RowTile<QT, D, kBwdThreads, 8> RTile;
     constexpr int QS = RTile::kStride;
-    constexpr int TS = TTile::kStride;
-    static_assert(QS == DkvLds<D>::QS && TS == DkvLds<D>::TS, "LDS layout mismatch");
+    static_assert(QS == DkvLds<D>::QS, "LDS layout mismatch");
     constexpr int KSTEPS = D / 16;
     constexpr int CB = D / 32;
 
@@ -305,18 +296,18 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
 
     RTile qtile;
     RTile gtile;
-    TTile qttile;
-    TTile gttile;
     float row_val = 0.0f;  // threads 0..63: lse * log2(e); threads 64..127: delta
+    const int ld_off = RTile::global_offset(tid);
+    const int st_off = RTile::lds_offset(tid);
 
     auto load_stage = [&](int it) {
         const int h = kvh * group + it / n_qt;
         const int q0 = (q_first + it % n_qt) * QT;
         const long long q_head = ((long long)b * g.q_heads + h) * T * D;
-        qtile.load(q + q_head, q0, T, tid);
-        gtile.load(d_out + q_head, q0, T, tid);
-        qttile.load(q + q_head, q0, T, tid);
-        gttile.load(d_out + q_head, q0, T, tid);
+        const __amdgpu_buffer_rsrc_t q_rsrc = make_head_rsrc(q + q_head, (long long)T * D * 2);
+        const __amdgpu_buffer_rsrc_t g_rsrc = make_head_rsrc(d_out + q_head, (long long)T * D * 2);
+        qtile.load(q_rsrc, ld_off, q0 * D * 2);
+        gtile.load(g_rsrc, ld_off, q0 * D * 2);
         if (tid < QT) {
             const int t = q0 + tid;
             row_val = t < T ? lse[b * lm.pack_stride + h * lm.head_stride + t] * kLog2e : __builtin_inff();
@@ -326,10 +317,8 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
         }
     };
     auto store_stage = [&](DkvLds<D>& st) {
-        qtile.store(st.q, tid);
-        gtile.store(st.g, tid);
-        qttile.store(st.qt, tid);
-        gttile.store(st.gt, tid);
+        qtile.store(st.q, st_off);
+        gtile.store(st.g, st_off);
         if (tid < QT)
             st.lse2[tid] = row_val;
         else if (tid < 2 * QT)
@@ -343,7 +332,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
     __syncthreads();
 
     const int r_off = row_perm(n) * QS + gh * 8;
-    const int t_off = n * TS + gh * 8;
+    const int t_off = transposed_read_offset(lane, QS);
 
     for (int it = 0; it < n_iter; ++it) {
         const bool more = it + 1 < n_iter;
@@ -413,9 +402,9 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
             for (int c2i = 0; c2i < 2; ++c2i) {
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
-                    const u32x4 ag = lds_read128(&st.gt[cb * 32 * TS + t_off + qb * 32 + c2i * 16]);
+                    const u32x4 ag = lds_read_transposed(&st.g[t_off + (qb * 32 + c2i * 16) * QS + cb * 32], QS);
                     dv_acc[cb] = E::mfma(ag, pf[c2i], dv_acc[cb]);
-                    const u32x4 aq = lds_read128(&st.qt[cb * 32 * TS + t_off + qb * 32 + c2i * 16]);
+                    const u32x4 aq = lds_read_transposed(&st.q[t_off + (qb * 32 + c2i * 16) * QS + cb * 32], QS);
                     dk_acc[cb] = E::mfma(aq, dsf[c2i], dk_acc[cb]);
                 }
             }

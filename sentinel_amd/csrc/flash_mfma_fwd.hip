@@ -2,13 +2,17 @@
 //
 // Replaces CudaFlashAttentionForwardWmma64Entry (sentinel/NeuralNet/Cuda/CudaFlashAttention.cu:1105-1266):
 // same result (O and per-query LSE = max + ln(sum), natural log of the scaled scores), different design:
-//   * tensors are [B, H, T, D] 16-bit, so every global access is a coalesced 128-bit (K, Q) or
-//     full-row dword (V) load; nothing is converted or gathered per tile;
+//   * tensors are [B, H, T, D] 16-bit, so every global access is a coalesced 128-bit buffer load with
+//     a loop-invariant vector offset (the hardware range check zero-fills rows past T); nothing is
+//     converted or gathered per tile;
 //   * a workgroup of 4 wavefronts owns 128 queries (32 per wavefront) and walks 64-key tiles;
-//     Q stays in registers for the whole kernel, K and V^T tiles are double-buffered in LDS and the
-//     next tile's global loads are in flight while the current one is multiplied;
+//     Q stays in registers for the whole kernel, K and V tiles are double-buffered in LDS (row-major)
+//     and the next tile's global loads are in flight while the current one is multiplied;
 //   * S^T = K Q^T, so a lane owns one query: the online-softmax max / sum are in-register plus one
-//     v_permlane32_swap, and P^T feeds the P V product from registers (no LDS round trip);
+//     v_permlane32_swap, and P^T feeds the P V product from registers (no LDS round trip); V^T is read
+//     out of the row-major V tile with transposing LDS reads;
+//   * the running maximum is only raised (and O rescaled) when a row's maximum grows by more than 2^8,
+//     which is exact and keeps P within the 16-bit range;
 //   * key tiles above the diagonal are skipped; only tiles that cross it are masked;
 //   * grouped-query attention reads the shared K/V head in place.
 #include "flash_common.h"
@@ -29,15 +33,15 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
                                                                    float* __restrict__ lse, RowMap lm, AttnGeom g,
                                                                    int q_tiles, int total_tiles) {
     constexpr int KT = kFwdKeyTile;
-    typedef RowTile<KT, D, kFwdThreads> KTile;
-    typedef TransposedTile<KT, D, kFwdThreads> VTile;
+    typedef RowTile<KT, D, kFwdThreads, 8> KTile;
+    typedef RowTile<KT, D, kFwdThreads, 16> VTile;
     constexpr int KS = KTile::kStride;
     constexpr int VS = VTile::kStride;
     constexpr int KSTEPS = D / 16;  // k-steps of the S^T product
     constexpr int CB = D / 32;      // 32-row blocks of O^T
 
     __shared__ __attribute__((aligned(16))) unsigned short k_lds[2][KT * KS];
-    __shared__ __attribute__((aligned(16))) unsigned short v_lds[2][D * VS];
+    __shared__ __attribute__((aligned(16))) unsigned short v_lds[2][KT * VS];
 
     // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of tiles so
     // that the q-tiles of one head (which stream the same K/V) share one L2.
@@ -74,12 +78,17 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     const int q_hi = min(T, (qt + 1) * kFwdQueryTile);        // one past the last query of the tile
     const int kv_tiles = CAUSAL ? (q_hi + KT - 1) / KT : (T + KT - 1) / KT;
 
+    const __amdgpu_buffer_rsrc_t k_rsrc = make_head_rsrc(kb, (long long)T * D * 2);
+    const __amdgpu_buffer_rsrc_t v_rsrc = make_head_rsrc(vb, (long long)T * D * 2);
+    const int ld_off = KTile::global_offset(tid);
+    const int k_st = KTile::lds_offset(tid);
+    const int v_st = VTile::lds_offset(tid);
     KTile kt;
     VTile vt;
-    kt.load(kb, 0, T, tid);
-    vt.load(vb, 0, T, tid);
-    kt.store(k_lds[0], tid);
-    vt.store(v_lds[0], tid);
+    kt.load(k_rsrc, ld_off, 0);
+    vt.load(v_rsrc, ld_off, 0);
+    kt.store(k_lds[0], k_st);
+    vt.store(v_lds[0], v_st);
     __syncthreads();
 
     f32x16 acc[CB];
@@ -92,14 +101,15 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     const float c2 = g.scale * kLog2e;
 
     const int k_off = row_perm(n) * KS + gh * 8;  // K operand read: row carried by D row n
-    const int v_off = n * VS + gh * 8;            // V^T operand read
+    const int v_off = transposed_read_offset(lane, VS);  // V^T operand read out of the row-major tile
+    const float raise_after = 8.0f;                // log2 units a row maximum may grow before O is rescaled
 
     for (int j = 0; j < kv_tiles; ++j) {
         const int buf = j & 1;
         const bool more = j + 1 < kv_tiles;
         if (more) {
-            kt.load(kb, (j + 1) * KT, T, tid);
-            vt.load(vb, (j + 1) * KT, T, tid);
+            kt.load(k_rsrc, ld_off, (j + 1) * KT * D * 2);
+            vt.load(v_rsrc, ld_off, (j + 1) * KT * D * 2);
         }
 
         const int key0 = j * KT;
@@ -136,9 +146,18 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
 #pragma unroll
             for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[1][i]);
             mx = half_max(mx);
-            const float m_new = fmaxf(m_run, mx);
-            const float mc = m_new * c2;
-            const float alpha = __builtin_amdgcn_exp2f(m_run * c2 - mc);
+            // raise the reference maximum only when some row outgrew it by more than 2^raise_after
+            if (__any((mx - m_run) * c2 > raise_after)) {
+                const float m_new = fmaxf(m_run, mx);
+                const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c2);
+                l_run *= alpha;
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[cb][i] *= alpha;
+                m_run = m_new;
+            }
+            const float mc = m_run * c2;
 
             float psum = 0.0f;
             u32x4 pf[4];  // P^T as B operand, four 16-key k-steps
@@ -155,28 +174,21 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
                     }
                 }
             }
-            l_run = l_run * alpha + psum;
-            if (__any(m_new > m_run)) {
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[cb][i] *= alpha;
-            }
-            m_run = m_new;
+            l_run += psum;
 
 #pragma unroll
             for (int c4 = 0; c4 < 4; ++c4) {
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
-                    const u32x4 a = lds_read128(&v_lds[buf][cb * 32 * VS + v_off + c4 * 16]);
+                    const u32x4 a = lds_read_transposed(&v_lds[buf][v_off + c4 * 16 * VS + cb * 32], VS);
                     acc[cb] = E::mfma(a, pf[c4], acc[cb]);
                 }
             }
         }
 
         if (more) {
-            kt.store(k_lds[buf ^ 1], tid);
-            vt.store(v_lds[buf ^ 1], tid);
+            kt.store(k_lds[buf ^ 1], k_st);
+            vt.store(v_lds[buf ^ 1], v_st);
         }
         __syncthreads();
     }

@@ -100,88 +100,71 @@ __device__ __forceinline__ u32x4 lds_read128(const unsigned short* p) { return *
 __device__ __forceinline__ void lds_write128(unsigned short* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 
 // ---------------------------------------------------------------------------------------------
-// Row-major tile: ROWS x D 16-bit elements of a [.., T, D] tensor -> registers -> LDS[row][D + 8].
-// The 8-element pad makes the 128-bit operand reads of 16 consecutive rows hit 64 distinct banks.
+// Global -> LDS staging of a ROWS x D tile of 16-bit elements out of a row-major [T, D] head.
+//
+// Loads are raw buffer loads: the resource describes exactly one head (T * D * 2 bytes), the per-thread
+// byte offset inside a tile is a loop-invariant VGPR and the tile's position is one SGPR, so walking the
+// sequence costs no vector address arithmetic and rows past T come back as zeros from the hardware's
+// range check (no branches).  LDS rows are padded by PAD elements.
 // ---------------------------------------------------------------------------------------------
-template <int ROWS, int D, int THREADS>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_head_rsrc(const unsigned short* base, long long bytes) {
+    const int limit = bytes > 0x7fffffffLL ? 0x7fffffff : (int)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned short*>(base), 0, limit, 0x00020000);
+}
+
+template <int ROWS, int D, int THREADS, int PAD>
 struct RowTile {
-    static constexpr int kStride = D + 8;
+    static constexpr int kStride = D + PAD;
     static constexpr int kChunksPerRow = D / 8;
     static constexpr int kIters = ROWS * kChunksPerRow / THREADS;
+    static constexpr int kRowsPerIter = THREADS / kChunksPerRow;
     static_assert(ROWS * kChunksPerRow % THREADS == 0, "tile must divide evenly over the workgroup");
     u32x4 regs[kIters];
 
-    // rows >= row_limit are zero-filled
-    __device__ __forceinline__ void load(const unsigned short* base, int row0, int row_limit, int tid) {
+    // byte offset of this thread's first chunk inside a tile / element offset of its LDS slot
+    static __device__ __forceinline__ int global_offset(int tid) { return ((tid / kChunksPerRow) * D + (tid % kChunksPerRow) * 8) * 2; }
+    static __device__ __forceinline__ int lds_offset(int tid) { return (tid / kChunksPerRow) * kStride + (tid % kChunksPerRow) * 8; }
+
+    // tile_bytes = first row of the tile * D * 2 (wavefront-uniform)
+    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rsrc, int thread_offset, int tile_bytes) {
 #pragma unroll
-        for (int it = 0; it < kIters; ++it) {
-            const int id = it * THREADS + tid;
-            const int r = id / kChunksPerRow;
-            const int cc = id % kChunksPerRow;
-            const int row = row0 + r;
-            u32x4 x = {0u, 0u, 0u, 0u};
-            if (row < row_limit) x = *reinterpret_cast<const u32x4*>(base + (long long)row * D + cc * 8);
-            regs[it] = x;
-        }
+        for (int it = 0; it < kIters; ++it)
+            regs[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, thread_offset + it * kRowsPerIter * D * 2, tile_bytes, 0);
     }
-    __device__ __forceinline__ void store(unsigned short* lds, int tid) const {
+    __device__ __forceinline__ void store(unsigned short* lds, int thread_lds_offset) const {
 #pragma unroll
-        for (int it = 0; it < kIters; ++it) {
-            const int id = it * THREADS + tid;
-            const int r = id / kChunksPerRow;
-            const int cc = id % kChunksPerRow;
-            lds_write128(lds + r * kStride + cc * 8, regs[it]);
-        }
+        for (int it = 0; it < kIters; ++it) lds_write128(lds + thread_lds_offset + it * kRowsPerIter * kStride, regs[it]);
     }
 };
 
 // ---------------------------------------------------------------------------------------------
-// Transposed tile: ROWS x D elements of a [.., T, D] tensor -> LDS[c][ROWS + 8] (token-contiguous),
-// the orientation needed when the contraction runs over tokens.  Each thread reads two adjacent
-// columns of eight consecutive rows (one dword per row, a full wavefront covers whole rows) and
-// regroups them in registers into two 8-token runs.
+// A operand whose contraction runs over the ROWS (tokens) of a row-major LDS tile: the transposed view
+// tile^T[col][token], read with ds_read_b64_tr_b16.  Within a 16-lane group that instruction returns to
+// lane i the 4 x 16-bit values {element i%4 of the 8 bytes addressed by lane 4j + i/4, j = 0..3}; with
+// lane i addressing tile[t0 + i/4][c0 + 4*(i%4) ..] lane i therefore receives tile[t0 .. t0+3][c0 + i]:
+// four consecutive tokens of one column.  Two reads give the 8 tokens of this lane-half.
+//   lane groups: lanes 0-15 -> columns c0..c0+15, lanes 16-31 -> c0+16..c0+31 (operand rows n = lane % 32),
+//   lanes 32-63 the same columns for the second half of the contraction (tokens + 8).
 // ---------------------------------------------------------------------------------------------
-template <int ROWS, int D, int THREADS>
-struct TransposedTile {
-    static constexpr int kStride = ROWS + 8;
-    static constexpr int kColPairs = D / 2;
-    static constexpr int kGroupsPerPass = THREADS / kColPairs;
-    static constexpr int kIters = (ROWS / 8) / kGroupsPerPass;
-    static_assert((ROWS / 8) % kGroupsPerPass == 0 && kIters >= 1, "tile must divide evenly over the workgroup");
-    unsigned regs[kIters][8];
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
-    __device__ __forceinline__ void load(const unsigned short* base, int row0, int row_limit, int tid) {
-        const int c2 = tid % kColPairs;
-        const int kg = tid / kColPairs;
-#pragma unroll
-        for (int it = 0; it < kIters; ++it) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int row = row0 + (it * kGroupsPerPass + kg) * 8 + e;
-                unsigned x = 0u;
-                if (row < row_limit) x = *reinterpret_cast<const unsigned*>(base + (long long)row * D + 2 * c2);
-                regs[it][e] = x;
-            }
-        }
-    }
-    __device__ __forceinline__ void store(unsigned short* lds, int tid) const {
-        const int c2 = tid % kColPairs;
-        const int kg = tid / kColPairs;
-#pragma unroll
-        for (int it = 0; it < kIters; ++it) {
-            u32x4 even, odd;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                // {S0 = later token, S1 = earlier token}: bytes 0-3 come from S1, 4-7 from S0
-                even[j] = __builtin_amdgcn_perm(regs[it][2 * j + 1], regs[it][2 * j], 0x05040100u);
-                odd[j] = __builtin_amdgcn_perm(regs[it][2 * j + 1], regs[it][2 * j], 0x07060302u);
-            }
-            const int tok = (it * kGroupsPerPass + kg) * 8;
-            lds_write128(lds + (2 * c2) * kStride + tok, even);
-            lds_write128(lds + (2 * c2 + 1) * kStride + tok, odd);
-        }
-    }
-};
+__device__ __forceinline__ int transposed_read_offset(int lane, int stride) {
+    const int i = lane & 15;
+    const int column_block = (lane >> 4) & 1;
+    const int gh = lane >> 5;
+    return (gh * 8 + (i >> 2)) * stride + column_block * 16 + 4 * (i & 3);
+}
+
+// tile_at = tile + transposed_read_offset + t0 * stride + c0
+__device__ __forceinline__ u32x4 lds_read_transposed(const unsigned short* tile_at, int stride) {
+    typedef s16x4_t __attribute__((address_space(3))) * lds_ptr;
+    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at));
+    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at + 4 * stride));
+    const u32x2 a = __builtin_bit_cast(u32x2, lo);
+    const u32x2 b = __builtin_bit_cast(u32x2, hi);
+    u32x4 r = {a[0], a[1], b[0], b[1]};
+    return r;
+}
 
 }  // namespace sentinel_hip
 #endif
