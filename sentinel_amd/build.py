@@ -21,7 +21,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hi
 
 def _compile(src):
     obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC] + FLAGS + os.environ.get("SENTINEL_HIPCC_EXTRA", "").split() + ["-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)

@@ -20,6 +20,8 @@
 #include "flash_common.h"
 #include "mfma_tile.h"
 
+#include <type_traits>
+
 namespace sentinel_hip {
 namespace {
 
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     const int T = g.seq_len;
 
     const int tid = threadIdx.x;
-    const int wave = tid / 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);  // wavefront-uniform by construction; tell the compiler
     const int lane = tid % 64;
     const int n = lane % 32;
     const int gh = lane / 32;
@@ -109,8 +111,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
         gf[ks] = *reinterpret_cast<const u32x4*>(d_out + q_head + (long long)qload * D + ks * 16 + gh * 8);
     }
     const float c2 = g.scale * kLog2e;
-    const float lse2 = lse[b * lm.pack_stride + h * lm.head_stride + qload] * kLog2e;
-    const float dl = delta[(long long)h * g.packs * T + (long long)b * T + qload];
+    const float lse2_raw = lse[b * lm.pack_stride + h * lm.head_stride + qload];
+    float dl = delta[(long long)h * g.packs * T + (long long)b * T + qload];
 
     const int q_hi = min(T, (qt + 1) * kDqQueryTile);
     const int kv_tiles = CAUSAL ? (q_hi + KT - 1) / KT : (T + KT - 1) / KT;
@@ -125,6 +127,14 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     vtile.load(v_rsrc, ld_off, 0);
     ktile.store(k_lds[0], st_off);
     vtile.store(v_lds[0], st_off);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        pin_loaded(qf[ks]);
+        pin_loaded(gf[ks]);
+    }
+    float lse2 = lse2_raw * kLog2e;
+    pin_loaded(lse2);
+    pin_loaded(dl);
     __syncthreads();
 
     f32x16 acc[CB];
@@ -224,7 +234,8 @@ constexpr int kDkvQueryTile = 64;
 template <int D>
 struct DkvLds {
     static constexpr int QT = kDkvQueryTile;
-    static constexpr int QS = D + 8;
+    static constexpr int kPad = 16;  // row pad (elements) that suits both the 128-bit row reads and the transposed reads
+    static constexpr int QS = D + kPad;
     unsigned short q[QT * QS];
     unsigned short g[QT * QS];
     float lse2[QT];
@@ -238,7 +249,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
     int total_tiles) {
     constexpr int QT = kDkvQueryTile;
-    typedef RowTile<QT, D, kBwdThreads, 8> RTile;
+    typedef RowTile<QT, D, kBwdThreads, DkvLds<D>::kPad> RTile;
     constexpr int QS = RTile::kStride;
     static_assert(QS == DkvLds<D>::QS, "LDS layout mismatch");
     constexpr int KSTEPS = D / 16;
@@ -258,7 +269,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
     const int T = g.seq_len;
 
     const int tid = threadIdx.x;
-    const int wave = tid / 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);  // wavefront-uniform by construction; tell the compiler
     const int lane = tid % 64;
     const int n = lane % 32;
     const int gh = lane / 32;
@@ -296,122 +307,177 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
 
     RTile qtile;
     RTile gtile;
-    float row_val = 0.0f;  // threads 0..63: lse * log2(e); threads 64..127: delta
+    float row_val = 0.0f;  // threads 0..63: lse; threads 64..127: delta
     const int ld_off = RTile::global_offset(tid);
     const int st_off = RTile::lds_offset(tid);
 
+    // threads 0..63 fetch lse, 64..127 delta of the stage's queries (the upper half of the workgroup repeats
+    // them); the row load is issued before the tile loads so that waiting for it never waits for those
+    const int row_slot = tid % QT;
+    const bool row_is_delta = (tid / QT) & 1;
     auto load_stage = [&](int it) {
         const int h = kvh * group + it / n_qt;
         const int q0 = (q_first + it % n_qt) * QT;
         const long long q_head = ((long long)b * g.q_heads + h) * T * D;
+        const int t = min(q0 + row_slot, T - 1);
+        const float* row_src = row_is_delta ? delta + (long long)h * g.packs * T + (long long)b * T
+                                            : lse + b * lm.pack_stride + h * lm.head_stride;
+        row_val = row_src[t];
         const __amdgpu_buffer_rsrc_t q_rsrc = make_head_rsrc(q + q_head, (long long)T * D * 2);
         const __amdgpu_buffer_rsrc_t g_rsrc = make_head_rsrc(d_out + q_head, (long long)T * D * 2);
         qtile.load(q_rsrc, ld_off, q0 * D * 2);
         gtile.load(g_rsrc, ld_off, q0 * D * 2);
-        if (tid < QT) {
-            const int t = q0 + tid;
-            row_val = t < T ? lse[b * lm.pack_stride + h * lm.head_stride + t] * kLog2e : __builtin_inff();
-        } else if (tid < 2 * QT) {
-            const int t = q0 + tid - QT;
-            row_val = t < T ? delta[(long long)h * g.packs * T + (long long)b * T + t] : 0.0f;
-        }
     };
-    auto store_stage = [&](DkvLds<D>& st) {
+    auto store_stage = [&](DkvLds<D>& st, int it) {
         qtile.store(st.q, st_off);
         gtile.store(st.g, st_off);
+        const int q0 = (q_first + it % n_qt) * QT;
+        const bool live = q0 + row_slot < T;
         if (tid < QT)
-            st.lse2[tid] = row_val;
+            st.lse2[row_slot] = live ? row_val * kLog2e : __builtin_inff();  // exp2(s - inf) = 0 for padded queries
         else if (tid < 2 * QT)
-            st.dl[tid - QT] = row_val;
+            st.dl[row_slot] = live ? row_val : 0.0f;
     };
 
-    if (n_iter > 0) {
-        load_stage(0);
-        store_stage(lds[0]);
+    // n_iter >= 1 always (the key tile's own queries)
+    load_stage(0);
+    store_stage(lds[0], 0);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        pin_loaded(kf[ks]);
+        pin_loaded(vf[ks]);
     }
     __syncthreads();
 
     const int r_off = row_perm(n) * QS + gh * 8;
     const int t_off = transposed_read_offset(lane, QS);
 
-    for (int it = 0; it < n_iter; ++it) {
-        const bool more = it + 1 < n_iter;
-        if (more) load_stage(it + 1);
-        DkvLds<D>& st = lds[it & 1];
-        const int q0 = (q_first + it % n_qt) * QT;
-
+    // P and dS of one 32-query block from its S and dP tiles (this lane: one key, 16 queries), rounded and
+    // packed as the B operands of the dV / dK products.  MASKED is only instantiated for stages that touch
+    // the causal diagonal or the end of the sequence, so the common case carries no compare / select.
+    auto softmax_backward = [&](auto masked_tag, const f32x16& s, const f32x16& dp, const DkvLds<D>& st, int qb, int q0b,
+                                u32x4 (&pf)[2], u32x4 (&dsf)[2]) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        float l2[16];
+        float dl[16];
 #pragma unroll
-        for (int qb = 0; qb < QT / 32; ++qb) {
-            const int q0b = q0 + qb * 32;
-            const bool skip = (CAUSAL && q0b + 31 < k0w) || q0b >= T;
-            if (skip) continue;
-            f32x16 s;
-            f32x16 dp;
+        for (int run = 0; run < 2; ++run)
+#pragma unroll
+            for (int part = 0; part < 2; ++part) {
+                const int base = qb * 32 + run * 16 + gh * 8 + part * 4;
+                const float4 a = *reinterpret_cast<const float4*>(&st.lse2[base]);
+                const float4 d4 = *reinterpret_cast<const float4*>(&st.dl[base]);
+                const int i0 = run * 8 + part * 4;
+                l2[i0] = a.x; l2[i0 + 1] = a.y; l2[i0 + 2] = a.z; l2[i0 + 3] = a.w;
+                dl[i0] = d4.x; dl[i0 + 1] = d4.y; dl[i0 + 2] = d4.z; dl[i0 + 3] = d4.w;
+            }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float p2[2];
+                float ds2[2];
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    const int i = half * 8 + 2 * e + w;
+                    float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -l2[i]));
+                    if (MASKED) {
+                        const int query = q0b + perm_row_of_reg(i, gh);
+                        if ((CAUSAL && key > query) || key_dead) p = 0.0f;
+                    }
+                    p2[w] = p;
+                    ds2[w] = p * (dp[i] - dl[i]);
+                }
+                pf[half][e] = E::pack2(p2[0], p2[1]);
+                dsf[half][e] = E::pack2(ds2[0], ds2[1]);
+            }
+        }
+    };
+
+    // One stage = NB 32-query blocks.  PIPELINED spells out a software pipeline for the instruction scheduler:
+    // region b runs the softmax-backward of block b on the vector ALU while the matrix pipe works on the
+    // dV / dK products of block b-1 and the S / dP products of block b+1.  Blocks entirely above the diagonal
+    // are not skipped (a few per workgroup): they are masked to zero instead, which keeps the code branch-free.
+    auto process_stage = [&](auto masked_tag, const DkvLds<D>& st, int q0) {
+        constexpr int NB = QT / 32;
+        f32x16 s[2];
+        f32x16 dp[2];
+        u32x4 pf[2][2];
+        u32x4 dsf[2][2];
+        auto scores = [&](int blk) {  // S and dP of block blk
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                s[i] = 0.0f;
-                dp[i] = 0.0f;
+                s[blk & 1][i] = 0.0f;
+                dp[blk & 1][i] = 0.0f;
             }
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
-                const u32x4 aq = lds_read128(&st.q[qb * 32 * QS + r_off + ks * 16]);
-                s = E::mfma(aq, kf[ks], s);
-                const u32x4 ag = lds_read128(&st.g[qb * 32 * QS + r_off + ks * 16]);
-                dp = E::mfma(ag, vf[ks], dp);
+                s[blk & 1] = E::mfma(lds_read128(&st.q[blk * 32 * QS + r_off + ks * 16]), kf[ks], s[blk & 1]);
+                dp[blk & 1] = E::mfma(lds_read128(&st.g[blk * 32 * QS + r_off + ks * 16]), vf[ks], dp[blk & 1]);
             }
-            // per-query lse and delta of the 16 queries this lane holds: two runs of eight
-            float l2[16];
-            float dl[16];
+        };
+        auto gradients = [&](int blk) {  // dV += dO^T P, dK += Q^T dS of block blk
 #pragma unroll
-            for (int run = 0; run < 2; ++run)
-#pragma unroll
-                for (int part = 0; part < 2; ++part) {
-                    const int base = qb * 32 + run * 16 + gh * 8 + part * 4;
-                    const float4 a = *reinterpret_cast<const float4*>(&st.lse2[base]);
-                    const float4 d4 = *reinterpret_cast<const float4*>(&st.dl[base]);
-                    const int i0 = run * 8 + part * 4;
-                    l2[i0] = a.x; l2[i0 + 1] = a.y; l2[i0 + 2] = a.z; l2[i0 + 3] = a.w;
-                    dl[i0] = d4.x; dl[i0 + 1] = d4.y; dl[i0 + 2] = d4.z; dl[i0 + 3] = d4.w;
-                }
-            const bool need_mask = CAUSAL && q0b < k0w + 31;
-            u32x4 pf[2];
-            u32x4 dsf[2];
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float p2[2];
-                    float ds2[2];
-#pragma unroll
-                    for (int w = 0; w < 2; ++w) {
-                        const int i = half * 8 + 2 * e + w;
-                        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -l2[i]));
-                        if (need_mask) {
-                            const int query = q0b + perm_row_of_reg(i, gh);
-                            if (key > query) p = 0.0f;
-                        }
-                        if (key_dead) p = 0.0f;
-                        p2[w] = p;
-                        ds2[w] = p * (dp[i] - dl[i]);
-                    }
-                    pf[half][e] = E::pack2(p2[0], p2[1]);
-                    dsf[half][e] = E::pack2(ds2[0], ds2[1]);
-                }
-            }
-#pragma unroll
-            for (int c2i = 0; c2i < 2; ++c2i) {
+            for (int c2i = 0; c2i < 2; ++c2i)
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
-                    const u32x4 ag = lds_read_transposed(&st.g[t_off + (qb * 32 + c2i * 16) * QS + cb * 32], QS);
-                    dv_acc[cb] = E::mfma(ag, pf[c2i], dv_acc[cb]);
-                    const u32x4 aq = lds_read_transposed(&st.q[t_off + (qb * 32 + c2i * 16) * QS + cb * 32], QS);
-                    dk_acc[cb] = E::mfma(aq, dsf[c2i], dk_acc[cb]);
+                    const u32x4 tg = lds_read_transposed(&st.g[t_off + (blk * 32 + c2i * 16) * QS + cb * 32], QS);
+                    dv_acc[cb] = E::mfma(tg, pf[blk & 1][c2i], dv_acc[cb]);
+                    const u32x4 tq = lds_read_transposed(&st.q[t_off + (blk * 32 + c2i * 16) * QS + cb * 32], QS);
+                    dk_acc[cb] = E::mfma(tq, dsf[blk & 1][c2i], dk_acc[cb]);
                 }
+        };
+#ifdef SENTINEL_DKDV_PIPELINED
+        scores(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk) {
+            softmax_backward(masked_tag, s[blk & 1], dp[blk & 1], st, blk, q0 + blk * 32, pf[blk & 1], dsf[blk & 1]);
+            if (blk > 0) gradients(blk - 1);
+            if (blk + 1 < NB) scores(blk + 1);
+#pragma unroll
+            for (int step = 0; step < 32; ++step) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // its LDS operand reads
+                __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // vector ALU work in its shadow
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
+        gradients(NB - 1);
+#else
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk) {
+            scores(blk);
+            softmax_backward(masked_tag, s[blk & 1], dp[blk & 1], st, blk, q0 + blk * 32, pf[blk & 1], dsf[blk & 1]);
+            gradients(blk);
+        }
+#endif
+    };
 
-        if (more) store_stage(lds[(it + 1) & 1]);
+    // one trip of the stage loop: prefetch the next stage, work on this one, publish the next one
+    auto stage_trip = [&](auto masked_tag, int it) {
+        const bool more = it + 1 < n_iter;
+        if (more) load_stage(it + 1);
+        process_stage(masked_tag, lds[it & 1], (q_first + it % n_qt) * QT);
+        if (more) store_stage(lds[(it + 1) & 1], it + 1);
         __syncthreads();
+    };
+
+    // Per query head of the group: the leading stages that touch this wavefront's causal diagonal (all stages if
+    // the key tile runs past the end of the sequence) take the masked code, the rest the unmasked code.  Two
+    // loops one after the other rather than a branch inside one loop, so the accumulators have one home.
+    {
+        int it = 0;
+        for (int gi = 0; gi < group; ++gi) {
+            const int head_end = (gi + 1) * n_qt;
+            int masked_end = it;
+            if (k0w + 31 >= T)
+                masked_end = head_end;
+            else if (CAUSAL)
+                masked_end = min(head_end, it + max(0, (k0w + 31 + QT - 1) / QT - q_first));
+            for (; it < masked_end; ++it) stage_trip(std::true_type{}, it);
+            for (; it < head_end; ++it) stage_trip(std::false_type{}, it);
+        }
     }
 
     if (!key_dead) {

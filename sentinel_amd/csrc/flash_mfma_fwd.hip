@@ -56,7 +56,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     const int T = g.seq_len;
 
     const int tid = threadIdx.x;
-    const int wave = tid / 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);  // wavefront-uniform by construction; tell the compiler
     const int lane = tid % 64;
     const int n = lane % 32;
     const int gh = lane / 32;
@@ -89,6 +89,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     vt.load(v_rsrc, ld_off, 0);
     kt.store(k_lds[0], k_st);
     vt.store(v_lds[0], v_st);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) pin_loaded(qf[ks]);
     __syncthreads();
 
     f32x16 acc[CB];

@@ -96,6 +96,13 @@ __device__ __forceinline__ float half_sum(float x) {
     return lo + hi;
 }
 
+// Makes a register value opaque at this point of the program: a global load feeding it must have been
+// issued and waited for before here.  Used on operand fragments that are loaded once and consumed inside
+// a loop: without it the compiler sinks the loads next to the loop and then guards their first use with
+// vmcnt waits that, on every later trip, drain the prefetch loads issued at the top of the same trip.
+__device__ __forceinline__ void pin_loaded(u32x4& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void pin_loaded(float& x) { asm volatile("" : "+v"(x)); }
+
 __device__ __forceinline__ u32x4 lds_read128(const unsigned short* p) { return *reinterpret_cast<const u32x4*>(p); }
 __device__ __forceinline__ void lds_write128(unsigned short* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 

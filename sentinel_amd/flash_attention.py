@@ -18,7 +18,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "lib", "libsentinel_hip_attn.so")
+# SENTINEL_HIP_ATTN_LIB points at another build of the same library (e.g. an experimental kernel variant)
+_LIB_PATH = os.environ.get("SENTINEL_HIP_ATTN_LIB") or os.path.join(_HERE, "lib", "libsentinel_hip_attn.so")
 
 OK, INVALID_ARGUMENT, UNSUPPORTED, RUNTIME = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
