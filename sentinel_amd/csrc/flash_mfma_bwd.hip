@@ -234,7 +234,7 @@ constexpr int kDkvQueryTile = 64;
 template <int D>
 struct DkvLds {
     static constexpr int QT = kDkvQueryTile;
-    static constexpr int kPad = 16;  // row pad (elements) that suits both the 128-bit row reads and the transposed reads
+    static constexpr int kPad = 8;  // row pad (elements): conflict-free for the 128-bit row reads and the transposed reads
     static constexpr int QS = D + kPad;
     unsigned short q[QT * QS];
     unsigned short g[QT * QS];
@@ -358,19 +358,27 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
     auto softmax_backward = [&](auto masked_tag, const f32x16& s, const f32x16& dp, const DkvLds<D>& st, int qb, int q0b,
                                 u32x4 (&pf)[2], u32x4 (&dsf)[2]) {
         constexpr bool MASKED = decltype(masked_tag)::value;
+        // lse and delta of the 16 queries this lane holds: rows 16*run + 8*gh + sigma(e), e = 0..7 (see mfma_tile.h)
         float l2[16];
         float dl[16];
 #pragma unroll
-        for (int run = 0; run < 2; ++run)
+        for (int run = 0; run < 2; ++run) {
+            float lrow[8];
+            float drow[8];
 #pragma unroll
             for (int part = 0; part < 2; ++part) {
                 const int base = qb * 32 + run * 16 + gh * 8 + part * 4;
                 const float4 a = *reinterpret_cast<const float4*>(&st.lse2[base]);
                 const float4 d4 = *reinterpret_cast<const float4*>(&st.dl[base]);
-                const int i0 = run * 8 + part * 4;
-                l2[i0] = a.x; l2[i0 + 1] = a.y; l2[i0 + 2] = a.z; l2[i0 + 3] = a.w;
-                dl[i0] = d4.x; dl[i0 + 1] = d4.y; dl[i0 + 2] = d4.z; dl[i0 + 3] = d4.w;
+                lrow[part * 4] = a.x; lrow[part * 4 + 1] = a.y; lrow[part * 4 + 2] = a.z; lrow[part * 4 + 3] = a.w;
+                drow[part * 4] = d4.x; drow[part * 4 + 1] = d4.y; drow[part * 4 + 2] = d4.z; drow[part * 4 + 3] = d4.w;
             }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                l2[run * 8 + e] = lrow[(e & 3) * 2 + (e >> 2)];
+                dl[run * 8 + e] = drow[(e & 3) * 2 + (e >> 2)];
+            }
+        }
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
 #pragma unroll

@@ -34,7 +34,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
                                                                    int q_tiles, int total_tiles) {
     constexpr int KT = kFwdKeyTile;
     typedef RowTile<KT, D, kFwdThreads, 8> KTile;
-    typedef RowTile<KT, D, kFwdThreads, 16> VTile;
+    typedef RowTile<KT, D, kFwdThreads, 8> VTile;
     constexpr int KS = KTile::kStride;
     constexpr int VS = VTile::kStride;
     constexpr int KSTEPS = D / 16;  // k-steps of the S^T product

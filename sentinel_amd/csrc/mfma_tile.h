@@ -11,10 +11,13 @@
 // in-register plus a single exchange between lane and lane+32.
 //
 // To turn a D result straight into the B operand of the next product (contraction over its rows), the
-// rows are loaded in the order row_perm(): D row index m then carries matrix row
-//   16*(m/16) + 8*((m/4)%2) + 4*((m/8)%2) + m%4,
-// which makes registers 0..7 of lane-half g hold rows 8g..8g+7 and registers 8..15 rows 16+8g..16+8g+7:
-// exactly the "contraction indices 8g..8g+7" packing of a B operand, for two consecutive k-steps.
+// rows of the first product are loaded in the order row_perm(): D row index m then carries matrix row
+// row_perm(m), chosen so that registers 0..7 of lane-half g hold rows 8g + {0,2,4,6,1,3,5,7} and registers
+// 8..15 the same rows + 16: the packing of a B operand for two consecutive k-steps whose contraction
+// index 8g + e stands for row 8g + sigma(e), sigma = {0,2,4,6,1,3,5,7}.  The matching A operand of the
+// second product is read with two transposing LDS reads that fetch the even and the odd rows of the
+// lane-half (lds_read_transposed); rows two apart is what keeps those reads free of bank conflicts with
+// the same 8-element row pad that suits the 128-bit row reads.
 #ifndef SENTINEL_HIP_MFMA_TILE_H
 #define SENTINEL_HIP_MFMA_TILE_H
 
@@ -62,13 +65,15 @@ struct Fp16 {
     }
 };
 
-// Matrix row carried by D row index m (see the header comment).
+// Matrix row carried by D row index m = 8a + 4g + r (see the header comment): 16*(a/2) + 8g + 2r + a%2.
 __device__ __forceinline__ int row_perm(int m) {
-    return (m & 16) | (((m >> 2) & 1) << 3) | (((m >> 3) & 1) << 2) | (m & 3);
+    return (m & 16) | (((m >> 2) & 1) << 3) | ((m & 3) << 1) | ((m >> 3) & 1);
 }
 
 // Row (within a 32-row block) held by D register i of lane-half g when the rows were loaded through row_perm.
-__device__ __forceinline__ int perm_row_of_reg(int i, int g) { return ((i >> 3) << 4) | (g << 3) | (i & 7); }
+__device__ __forceinline__ int perm_row_of_reg(int i, int g) {
+    return ((i >> 3) << 4) | (g << 3) | ((i & 3) << 1) | ((i >> 2) & 1);
+}
 
 // Plain D layout row of register i.
 __device__ __forceinline__ int plain_row_of_reg(int i, int g) { return ((i >> 2) << 3) | (g << 2) | (i & 3); }
@@ -148,8 +153,9 @@ struct RowTile {
 // A operand whose contraction runs over the ROWS (tokens) of a row-major LDS tile: the transposed view
 // tile^T[col][token], read with ds_read_b64_tr_b16.  Within a 16-lane group that instruction returns to
 // lane i the 4 x 16-bit values {element i%4 of the 8 bytes addressed by lane 4j + i/4, j = 0..3}; with
-// lane i addressing tile[t0 + i/4][c0 + 4*(i%4) ..] lane i therefore receives tile[t0 .. t0+3][c0 + i]:
-// four consecutive tokens of one column.  Two reads give the 8 tokens of this lane-half.
+// lane i addressing tile[t0 + 2*(i/4)][c0 + 4*(i%4) ..] lane i therefore receives
+// tile[t0 + {0,2,4,6}][c0 + i]: the even tokens of one column; a second read one row further gives the
+// odd ones.  Together: contraction elements e = 0..7 of this lane-half = tokens t0 + sigma(e).
 //   lane groups: lanes 0-15 -> columns c0..c0+15, lanes 16-31 -> c0+16..c0+31 (operand rows n = lane % 32),
 //   lanes 32-63 the same columns for the second half of the contraction (tokens + 8).
 // ---------------------------------------------------------------------------------------------
@@ -159,16 +165,16 @@ __device__ __forceinline__ int transposed_read_offset(int lane, int stride) {
     const int i = lane & 15;
     const int column_block = (lane >> 4) & 1;
     const int gh = lane >> 5;
-    return (gh * 8 + (i >> 2)) * stride + column_block * 16 + 4 * (i & 3);
+    return (gh * 8 + 2 * (i >> 2)) * stride + column_block * 16 + 4 * (i & 3);
 }
 
 // tile_at = tile + transposed_read_offset + t0 * stride + c0
 __device__ __forceinline__ u32x4 lds_read_transposed(const unsigned short* tile_at, int stride) {
     typedef s16x4_t __attribute__((address_space(3))) * lds_ptr;
-    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at));
-    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at + 4 * stride));
-    const u32x2 a = __builtin_bit_cast(u32x2, lo);
-    const u32x2 b = __builtin_bit_cast(u32x2, hi);
+    const s16x4_t even = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at));
+    const s16x4_t odd = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at + stride));
+    const u32x2 a = __builtin_bit_cast(u32x2, even);
+    const u32x2 b = __builtin_bit_cast(u32x2, odd);
     u32x4 r = {a[0], a[1], b[0], b[1]};
     return r;
 }
