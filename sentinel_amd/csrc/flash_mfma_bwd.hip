@@ -402,10 +402,8 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
         }
     };
 
-    // One stage = NB 32-query blocks.  PIPELINED spells out a software pipeline for the instruction scheduler:
-    // region b runs the softmax-backward of block b on the vector ALU while the matrix pipe works on the
-    // dV / dK products of block b-1 and the S / dP products of block b+1.  Blocks entirely above the diagonal
-    // are not skipped (a few per workgroup): they are masked to zero instead, which keeps the code branch-free.
+    // One stage = NB 32-query blocks.  Blocks entirely above the diagonal are not skipped (a few per
+    // workgroup): they are masked to zero instead, which keeps the stage body free of branches.
     auto process_stage = [&](auto masked_tag, const DkvLds<D>& st, int q0) {
         constexpr int NB = QT / 32;
         f32x16 s[2];
@@ -435,31 +433,12 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
                     dk_acc[cb] = E::mfma(tq, dsf[blk & 1][c2i], dk_acc[cb]);
                 }
         };
-#ifdef SENTINEL_DKDV_PIPELINED
-        scores(0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int blk = 0; blk < NB; ++blk) {
-            softmax_backward(masked_tag, s[blk & 1], dp[blk & 1], st, blk, q0 + blk * 32, pf[blk & 1], dsf[blk & 1]);
-            if (blk > 0) gradients(blk - 1);
-            if (blk + 1 < NB) scores(blk + 1);
-#pragma unroll
-            for (int step = 0; step < 32; ++step) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // its LDS operand reads
-                __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // vector ALU work in its shadow
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        gradients(NB - 1);
-#else
 #pragma unroll
         for (int blk = 0; blk < NB; ++blk) {
             scores(blk);
             softmax_backward(masked_tag, s[blk & 1], dp[blk & 1], st, blk, q0 + blk * 32, pf[blk & 1], dsf[blk & 1]);
             gradients(blk);
         }
-#endif
     };
 
     // one trip of the stage loop: prefetch the next stage, work on this one, publish the next one
