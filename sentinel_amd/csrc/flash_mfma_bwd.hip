@@ -71,13 +71,15 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                                                                   unsigned short* __restrict__ dq, RowMap lm, AttnGeom g,
                                                                   int q_tiles, int total_tiles) {
     constexpr int KT = kDqKeyTile;
-    typedef RowTile<KT, D, kBwdThreads, 8> RTile;
-    constexpr int KS = RTile::kStride;
+    typedef DirectTile<KT, D, kBwdThreads> Tile;
     constexpr int KSTEPS = D / 16;
     constexpr int CB = D / 32;
 
-    __shared__ __attribute__((aligned(16))) unsigned short k_lds[2][KT * KS];
-    __shared__ __attribute__((aligned(16))) unsigned short v_lds[2][KT * KS];
+    // two stages of (K, V) tiles; separate arrays so that loads into one stage are known not to alias reads of the other
+    __shared__ __attribute__((aligned(16))) unsigned short k_lds0[Tile::kElems];
+    __shared__ __attribute__((aligned(16))) unsigned short v_lds0[Tile::kElems];
+    __shared__ __attribute__((aligned(16))) unsigned short k_lds1[Tile::kElems];
+    __shared__ __attribute__((aligned(16))) unsigned short v_lds1[Tile::kElems];
 
     const int per_xcd = (int)gridDim.x / 8;
     const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
@@ -119,14 +121,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 
     const __amdgpu_buffer_rsrc_t k_rsrc = make_head_rsrc(kb, (long long)T * D * 2);
     const __amdgpu_buffer_rsrc_t v_rsrc = make_head_rsrc(vb, (long long)T * D * 2);
-    const int ld_off = RTile::global_offset(tid);
-    const int st_off = RTile::lds_offset(tid);
-    RTile ktile;
-    RTile vtile;
-    ktile.load(k_rsrc, ld_off, 0);
-    vtile.load(v_rsrc, ld_off, 0);
-    ktile.store(k_lds[0], st_off);
-    vtile.store(v_lds[0], st_off);
+    const int ld_off = Tile::global_offset(tid);
+    Tile::issue(k_rsrc, k_lds0, ld_off, 0, wave);
+    Tile::issue(v_rsrc, v_lds0, ld_off, 0, wave);
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
         pin_loaded(qf[ks]);
@@ -135,6 +132,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     float lse2 = lse2_raw * kLog2e;
     pin_loaded(lse2);
     pin_loaded(dl);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the first tiles have landed in LDS
     __syncthreads();
 
     f32x16 acc[CB];
@@ -143,15 +141,17 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[cb][i] = 0.0f;
 
-    const int k_off = row_perm(n) * KS + gh * 8;
-    const int t_off = transposed_read_offset(lane, KS);
+    const int k_off = Tile::row_read_base(row_perm(n), gh);
+    const int t_even = Tile::transposed_read_base(lane, 0);
+    const int t_odd = Tile::transposed_read_base(lane, 1);
 
-    for (int j = 0; j < kv_tiles; ++j) {
-        const int buf = j & 1;
+    // one trip over tile j held in (kt, vt); the next tile streams into (kt_next, vt_next) meanwhile
+    auto tile_trip = [&](int j, const unsigned short* kt, const unsigned short* vt, unsigned short* kt_next,
+                         unsigned short* vt_next) {
         const bool more = j + 1 < kv_tiles;
         if (more) {
-            ktile.load(k_rsrc, ld_off, (j + 1) * KT * D * 2);
-            vtile.load(v_rsrc, ld_off, (j + 1) * KT * D * 2);
+            Tile::issue(k_rsrc, kt_next, ld_off, (j + 1) * KT * D * 2, wave);
+            Tile::issue(v_rsrc, vt_next, ld_off, (j + 1) * KT * D * 2, wave);
         }
         const int key0 = j * KT;
         const bool skip = CAUSAL && key0 > q0w + 31;
@@ -169,9 +169,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                 }
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) {
-                    const u32x4 ak = lds_read128(&k_lds[buf][kbk * 32 * KS + k_off + ks * 16]);
+                    const u32x4 ak = lds_read128(kt + kbk * 32 * D + (k_off ^ (ks << 4)));
                     s = E::mfma(ak, qf[ks], s);
-                    const u32x4 av = lds_read128(&v_lds[buf][kbk * 32 * KS + k_off + ks * 16]);
+                    const u32x4 av = lds_read128(vt + kbk * 32 * D + (k_off ^ (ks << 4)));
                     dp = E::mfma(av, gf[ks], dp);
                 }
                 u32x4 dsf[2];
@@ -198,17 +198,20 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                 for (int half = 0; half < 2; ++half) {
 #pragma unroll
                     for (int cb = 0; cb < CB; ++cb) {
-                        const u32x4 a = lds_read_transposed(&k_lds[buf][t_off + (kbk * 32 + half * 16) * KS + cb * 32], KS);
+                        const int t0 = (kbk * 32 + half * 16) * D;
+                        const u32x4 a = lds_read_transposed_pair(kt + t0 + (t_even ^ (cb << 5)), kt + t0 + (t_odd ^ (cb << 5)));
                         acc[cb] = E::mfma(a, dsf[half], acc[cb]);
                     }
                 }
             }
         }
-        if (more) {
-            ktile.store(k_lds[buf ^ 1], st_off);
-            vtile.store(v_lds[buf ^ 1], st_off);
-        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's share of the next tile is in LDS
         __syncthreads();
+    };
+
+    for (int j = 0; j < kv_tiles; j += 2) {
+        tile_trip(j, k_lds0, v_lds0, k_lds1, v_lds1);
+        if (j + 1 < kv_tiles) tile_trip(j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
     }
 
     if (qrow < T) {

@@ -179,5 +179,59 @@ __device__ __forceinline__ u32x4 lds_read_transposed(const unsigned short* tile_
     return r;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Global -> LDS without passing through registers (buffer_load ... lds): each lane's 16 bytes land at
+// tile + 16 * (chunk index) in issue order, so the tile is unpadded; bank conflicts are avoided by an XOR
+// swizzle instead: the 16-byte chunk c of row r is kept at chunk position c ^ (r mod chunks_per_row),
+// which is applied on the global side (each lane fetches the chunk that belongs at its position).
+// Both operand read patterns stay conflict-free: 16 consecutive rows of one logical chunk hit 16 different
+// positions, and the transposed reads touch rows two apart whose chunk pairs fall on different positions.
+// ---------------------------------------------------------------------------------------------
+template <int ROWS, int D, int THREADS>
+struct DirectTile {
+    static constexpr int kChunksPerRow = D / 8;
+    static constexpr int kMask = kChunksPerRow - 1;
+    static constexpr int kIters = ROWS * kChunksPerRow / THREADS;
+    static constexpr int kRowsPerIter = THREADS / kChunksPerRow;
+    static constexpr int kElems = ROWS * D;
+    static_assert(ROWS * kChunksPerRow % THREADS == 0 && kRowsPerIter % kChunksPerRow == 0, "tile / swizzle period mismatch");
+
+    // byte offset (inside a tile of the head) of the chunk this thread fetches in pass 0
+    static __device__ __forceinline__ int global_offset(int tid) {
+        const int row = tid / kChunksPerRow;
+        const int pos = tid % kChunksPerRow;
+        return (row * D + ((pos ^ (row & kMask)) << 3)) * 2;
+    }
+    // tile_bytes = first row of the tile * D * 2; wave = wavefront index in the workgroup (both uniform)
+    static __device__ __forceinline__ void issue(__amdgpu_buffer_rsrc_t rsrc, unsigned short* lds_tile, int thread_offset,
+                                                 int tile_bytes, int wave) {
+        typedef __attribute__((address_space(3))) void* lds_void;
+#pragma unroll
+        for (int it = 0; it < kIters; ++it)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void)(lds_tile + (it * THREADS + wave * 64) * 8), 16,
+                                                     thread_offset + it * kRowsPerIter * D * 2, tile_bytes, 0, 0);
+    }
+    // element offset of this lane's 128-bit operand read of row `row` (k-step 0): xor (ks << 4) selects k-step ks
+    static __device__ __forceinline__ int row_read_base(int row, int gh) { return row * D + ((gh ^ (row & kMask)) << 3); }
+    // element offsets of this lane's two transposed reads (even / odd tokens) for token block 0, column block 0:
+    // add t0 * D for the token block (t0 a multiple of 16), xor (cb << 5) for column block cb
+    static __device__ __forceinline__ int transposed_read_base(int lane, int odd) {
+        const int i = lane & 15;
+        const int r = (lane >> 5) * 8 + 2 * (i >> 2) + odd;
+        const int chunk = ((lane >> 4) & 1) * 2 + ((i & 3) >> 1);
+        return r * D + ((chunk ^ (r & kMask)) << 3) + 4 * (i & 1);
+    }
+};
+
+__device__ __forceinline__ u32x4 lds_read_transposed_pair(const unsigned short* even_at, const unsigned short* odd_at) {
+    typedef s16x4_t __attribute__((address_space(3))) * lds_ptr;
+    const s16x4_t even = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(even_at));
+    const s16x4_t odd = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(odd_at));
+    const u32x2 a = __builtin_bit_cast(u32x2, even);
+    const u32x2 b = __builtin_bit_cast(u32x2, odd);
+    u32x4 r = {a[0], a[1], b[0], b[1]};
+    return r;
+}
+
 }  // namespace sentinel_hip
 #endif
