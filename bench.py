@@ -33,6 +33,9 @@ CONFIGS = {
 SEEDS = {"c1": 1, "c2": 2, "c3": 3, "c4": 4, "c5": 5, "nstar": 6}
 # algorithmic matrix products per kernel (units of B*H*T^2*d FLOPs, causal-halved)
 KERNEL_UNITS = {"fwd_mfma": 2.0, "dkdv_mfma": 4.0, "dq_mfma": 1.0, "fwd_f32": 2.0, "dkdv_f32": 4.0, "dq_f32": 1.0}
+# HBM bytes per launch at the target shape, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/nstar_b4_h32_t4096_d128_bf16_counters.txt (scaled by a plain copy kernel of known size: x2.0 / x1.0)
+MEASURED_TRAFFIC_BYTES = {("nstar", "fwd_mfma"): 5.47e8, ("nstar", "dkdv_mfma"): 8.10e8, ("nstar", "dq_mfma"): 6.76e8}
 
 
 def make_inputs(torch, name):
@@ -133,6 +136,9 @@ def main():
     ap.add_argument("--config", default="nstar", choices=sorted(CONFIGS))
     ap.add_argument("--cpu-heads", type=int, default=8, help="(batch, head) pairs in the CPU baseline sample; 0 = skip")
     ap.add_argument("--no-configs", action="store_true", help="skip the brief timing of the other configurations")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB -> 1 GiB elementwise copy kernel three times, so that a counter run "
+                         "(FETCH_SIZE / WRITE_SIZE) of this command holds a kernel of known traffic to scale by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only; attention shards over (batch, kv-head group) with no "
@@ -151,6 +157,13 @@ def main():
     ms_fwd = w.timed(w.forward, max(args.steps // 2, 1), 1)
     ms_bwd = w.timed(w.backward, max(args.steps // 2, 1), 1)
     kernels = w.kernel_times(args.steps)
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB read, 1 GiB written per launch
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     total_flops = 7.0 * w.unit_flops
     value = total_flops / (ms_step * 1e-3) / 1e12
     peak = PEAK_TFLOPS[w.dtype]
@@ -159,7 +172,7 @@ def main():
     dominant = max(counted, key=counted.get)
     achieved = KERNEL_UNITS[dominant] * w.unit_flops / (counted[dominant] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                "frac": achieved / peak, "traffic": None,
+                "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dominant)),
                 "kernel_ms": counted[dominant],
                 "algorithmic_flops_per_launch": KERNEL_UNITS[dominant] * w.unit_flops}
 
