@@ -27,6 +27,12 @@ namespace {
 
 constexpr int kBwdThreads = 256;
 
+// instruction classes of __builtin_amdgcn_sched_group_barrier
+constexpr int kSchedValu = 0x402;  // VALU and transcendental
+constexpr int kSchedMfma = 0x008;
+constexpr int kSchedDsRead = 0x100;
+constexpr int kOperandLead = 4;
+
 // ------------------------------------------------------------------------------------------------
 // D[h][b*T + t] = sum_c out * d_out  (16-bit inputs, fp32 sum)
 // ------------------------------------------------------------------------------------------------
@@ -145,18 +151,19 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     const int t_even = Tile::transposed_read_base(lane, 0);
     const int t_odd = Tile::transposed_read_base(lane, 1);
 
-    // one trip over tile j held in (kt, vt); the next tile streams into (kt_next, vt_next) meanwhile
-    auto tile_trip = [&](int j, const unsigned short* kt, const unsigned short* vt, unsigned short* kt_next,
+    // one trip over tile j held in (kt, vt); the next tile streams into (kt_next, vt_next) meanwhile.
+    // MASKED trips compare key against query per element; the others run the bare softmax-backward arithmetic.
+    auto tile_trip = [&](auto masked_tag, int j, const unsigned short* kt, const unsigned short* vt, unsigned short* kt_next,
                          unsigned short* vt_next) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
         const bool more = j + 1 < kv_tiles;
         if (more) {
             Tile::issue(k_rsrc, kt_next, ld_off, (j + 1) * KT * D * 2, wave);
             Tile::issue(v_rsrc, vt_next, ld_off, (j + 1) * KT * D * 2, wave);
         }
         const int key0 = j * KT;
-        const bool skip = CAUSAL && key0 > q0w + 31;
+        const bool skip = MASKED && CAUSAL && key0 > q0w + 31;
         if (!skip) {
-            const bool need_mask = CAUSAL ? (key0 + KT - 1 > q0w) : (key0 + KT > T);
             // two 32-key halves one after the other keeps the live score registers to one half
 #pragma unroll
             for (int kbk = 0; kbk < 2; ++kbk) {
@@ -167,51 +174,85 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                     s[i] = 0.0f;
                     dp[i] = 0.0f;
                 }
+                // program order = issue order wanted within each instruction class; the interleave of the classes
+                // is laid down by the scheduling groups at the end of the half
+                u32x4 ak[KSTEPS];
+                u32x4 av[KSTEPS];
 #pragma unroll
-                for (int ks = 0; ks < KSTEPS; ++ks) {
-                    const u32x4 ak = lds_read128(kt + kbk * 32 * D + (k_off ^ (ks << 4)));
-                    s = E::mfma(ak, qf[ks], s);
-                    const u32x4 av = lds_read128(vt + kbk * 32 * D + (k_off ^ (ks << 4)));
-                    dp = E::mfma(av, gf[ks], dp);
-                }
-                u32x4 dsf[2];
+                for (int ks = 0; ks < KSTEPS; ++ks) ak[ks] = lds_read128(kt + kbk * 32 * D + (k_off ^ (ks << 4)));
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
+                for (int ks = 0; ks < KSTEPS; ++ks) av[ks] = lds_read128(vt + kbk * 32 * D + (k_off ^ (ks << 4)));
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        float ds2[2];
+                for (int ks = 0; ks < KSTEPS; ++ks) s = E::mfma(ak[ks], qf[ks], s);
 #pragma unroll
-                        for (int w = 0; w < 2; ++w) {
-                            const int i = half * 8 + 2 * e + w;
-                            float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -lse2));
-                            if (need_mask) {
-                                const int key = key0 + kbk * 32 + perm_row_of_reg(i, gh);
-                                const bool dead = CAUSAL ? key > qrow : key >= T;
-                                if (dead) p = 0.0f;
-                            }
-                            ds2[w] = p * (dp[i] - dl);
-                        }
-                        dsf[half][e] = E::pack2(ds2[0], ds2[1]);
-                    }
-                }
+                for (int ks = 0; ks < KSTEPS; ++ks) dp = E::mfma(av[ks], gf[ks], dp);
+
+                u32x4 kt_frag[2][CB];
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
+                for (int half = 0; half < 2; ++half)
 #pragma unroll
                     for (int cb = 0; cb < CB; ++cb) {
                         const int t0 = (kbk * 32 + half * 16) * D;
-                        const u32x4 a = lds_read_transposed_pair(kt + t0 + (t_even ^ (cb << 5)), kt + t0 + (t_odd ^ (cb << 5)));
-                        acc[cb] = E::mfma(a, dsf[half], acc[cb]);
+                        kt_frag[half][cb] =
+                            lds_read_transposed_pair(kt + t0 + (t_even ^ (cb << 5)), kt + t0 + (t_odd ^ (cb << 5)));
+                    }
+                float p[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -lse2));
+                    if (MASKED) {
+                        const int key = key0 + kbk * 32 + perm_row_of_reg(i, gh);
+                        const bool dead = CAUSAL ? key > qrow : key >= T;
+                        if (dead) p[i] = 0.0f;
                     }
                 }
+                u32x4 dsf[2];
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int i = half * 8 + 2 * e;
+                        dsf[half][e] = E::pack2(p[i] * (dp[i] - dl), p[i + 1] * (dp[i + 1] - dl));
+                    }
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) acc[cb] = E::mfma(kt_frag[half][cb], dsf[half], acc[cb]);
+                }
+                if (!MASKED) {
+                    // S chain with its operand reads kOperandLead ahead, then the dP chain overlapped with exp(S) and
+                    // the transposed reads of the dQ operands, then the rest of the arithmetic, then the dQ chain
+                    __builtin_amdgcn_sched_group_barrier(kSchedDsRead, kOperandLead, 0);
+#pragma unroll
+                    for (int i = 0; i < 2 * KSTEPS - kOperandLead; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+                        if (i >= KSTEPS + 1) __builtin_amdgcn_sched_group_barrier(kSchedValu, 5, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < kOperandLead; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 2, 0);
+                        __builtin_amdgcn_sched_group_barrier(kSchedValu, 5, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's share of the next tile is in LDS
         __syncthreads();
     };
 
-    for (int j = 0; j < kv_tiles; j += 2) {
-        tile_trip(j, k_lds0, v_lds0, k_lds1, v_lds1);
-        if (j + 1 < kv_tiles) tile_trip(j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
+    // Tiles that end at or before the first query of the workgroup need no mask for any wavefront; keep the count
+    // even so that the masked tail starts on LDS stage 0 again.
+    const int bare_tiles = (CAUSAL ? min(kv_tiles, qt * (kDqQueryTile / KT)) : T / KT) & ~1;
+    for (int j = 0; j < bare_tiles; j += 2) {
+        tile_trip(std::false_type{}, j, k_lds0, v_lds0, k_lds1, v_lds1);
+        tile_trip(std::false_type{}, j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
+    }
+    for (int j = bare_tiles; j < kv_tiles; j += 2) {
+        tile_trip(std::true_type{}, j, k_lds0, v_lds0, k_lds1, v_lds1);
+        if (j + 1 < kv_tiles) tile_trip(std::true_type{}, j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
     }
 
     if (qrow < T) {
