@@ -6,10 +6,10 @@
 //     dV = P^T dO,  dK = dS^T Q,  dQ = dS K,          D = rowsum(dO o O)
 // but no atomics and no pre-zeroed outputs: the work is split into
 //   delta_mfma_kernel   D per query;
-//   dkdv_mfma_kernel    key-outer: a workgroup owns 128 keys of one K/V head, keeps K, V (as B operands)
-//                       and the dK^T, dV^T accumulators in registers, and streams the query tiles of every
-//                       query head of the group through LDS (grouped-query gradients are summed in
-//                       registers, replacing reduceKvHeadGradsInto, CudaCausalSelfAttention.cu:36-44);
+//   dkdv_split_kernel   key-outer: a workgroup owns 128 keys of one K/V head; per 32-key block one wavefront
+//                       keeps K (as B operand) and dV^T, a second one V and dK^T, and the query tiles of
+//                       every query head of the group stream through LDS (grouped-query gradients are summed
+//                       in registers, replacing reduceKvHeadGradsInto, CudaCausalSelfAttention.cu:36-44);
 //   dq_mfma_kernel      query-outer: a workgroup owns 128 queries, keeps Q, dO (as B operands) and dQ^T in
 //                       registers and streams K / V tiles through LDS (recomputing S and dP).
 // Tiles sit row-major in LDS; the products that contract over tokens (dV, dK, dQ) read their A operand out
@@ -269,68 +269,90 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     }
 }
 
-// ------------------------------------------------------------------------------------------------
-// dK, dV: key-outer
-// ------------------------------------------------------------------------------------------------
 constexpr int kDkvKeyTile = 128;
 constexpr int kDkvQueryTile = 64;
 
+// ------------------------------------------------------------------------------------------------
+// dK, dV with the work of a 32-key block split over two wavefronts (512 threads, two wavefronts per SIMD):
+//   score wavefront (waves 0..3):  S = Q K^T, P = exp2(S c - lse2), publishes P (16-bit) in LDS, dV^T += dO^T P
+//   grad  wavefront (waves 4..7):  dP - D = dO V^T - D (accumulator starts at -D), dS = P o (dP - D), dK^T += Q^T dS
+// The grad wavefronts run one stage behind the score wavefronts, so that P is always complete when it is
+// read and one workgroup barrier per stage is all the synchronisation there is: three tile stages rotate
+// (being filled / scored / back-propagated) and two P buffers alternate.  Each wavefront holds one operand
+// (K or V, 32 keys) and one accumulator (dV^T or dK^T) in registers: half the registers of doing both, which
+// is what lets two wavefronts share a SIMD and overlap one's exponentials with the other's matrix products.
+// ------------------------------------------------------------------------------------------------
+constexpr int kDkvSplitThreads = 512;
+
 template <int D>
-struct DkvLds {
+struct DkvSplitStage {
     static constexpr int QT = kDkvQueryTile;
-    static constexpr int kPad = 8;  // row pad (elements): conflict-free for the 128-bit row reads and the transposed reads
-    static constexpr int QS = D + kPad;
+    static constexpr int QS = D + 8;
     unsigned short q[QT * QS];
     unsigned short g[QT * QS];
-    float lse2[QT];
-    float dl[QT];
+    float nls[QT];  // -LSE / scale, in operand order (see stage_slot)
+    float ndl[QT];  // -D, same order
 };
 
+template <int D>
+struct DkvSplitLds {
+    DkvSplitStage<D> stage[3];
+    u32x4 p[2][4][2][2][64];  // [buffer][key block][32-query block][16-query half][lane]
+};
+
+// Position of query row r of a stage in the nls / ndl arrays: rows are kept in the order the score registers
+// of a lane hold them (the inverse of perm_row_of_reg: 16 * (r / 16) + 8 g + 4 a + j for r = 16 c + 4 j + 2 g + a),
+// so four 128-bit reads fill the 16 per-lane values in register order.
+__device__ __forceinline__ int stage_slot(int r) {
+    return (r & ~15) | (((r >> 1) & 1) << 3) | ((r & 1) << 2) | ((r >> 2) & 3);
+}
+
 template <typename E, int D, bool CAUSAL>
-__global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kernel(
+__global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
     int total_tiles) {
     constexpr int QT = kDkvQueryTile;
-    typedef RowTile<QT, D, kBwdThreads, DkvLds<D>::kPad> RTile;
+    typedef RowTile<QT, D, kDkvSplitThreads, 8> RTile;
     constexpr int QS = RTile::kStride;
-    static_assert(QS == DkvLds<D>::QS, "LDS layout mismatch");
+    static_assert(QS == DkvSplitStage<D>::QS, "LDS layout mismatch");
     constexpr int KSTEPS = D / 16;
     constexpr int CB = D / 32;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char dkv_smem[];
-    DkvLds<D>* lds = reinterpret_cast<DkvLds<D>*>(dkv_smem);  // two stages
+    DkvSplitLds<D>& lds = *reinterpret_cast<DkvSplitLds<D>*>(dkv_smem);
 
     const int per_xcd = (int)gridDim.x / 8;
     const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
     if (tile_id >= total_tiles) return;
     const int bkv = tile_id / k_tiles;
-    const int ktile = tile_id % k_tiles;  // under the causal mask the first key tiles see the most queries
+    const int ktile = tile_id % k_tiles;
     const int b = bkv / g.kv_heads;
     const int kvh = bkv % g.kv_heads;
     const int group = g.q_heads / g.kv_heads;
     const int T = g.seq_len;
 
     const int tid = threadIdx.x;
-    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);  // wavefront-uniform by construction; tell the compiler
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const bool grad_role = wave >= 4;
+    const int kblock = wave & 3;
     const int lane = tid % 64;
     const int n = lane % 32;
     const int gh = lane / 32;
 
     const long long kv_head = ((long long)b * g.kv_heads + kvh) * T * D;
-    const int k0w = ktile * kDkvKeyTile + wave * 32;
+    const int k0w = ktile * kDkvKeyTile + kblock * 32;
     const int key = k0w + n;
     const int kload = key < T ? key : T - 1;
     const bool key_dead = key >= T;
 
-    // K^T and V^T as B operands: column = key, contraction over head dims
-    u32x4 kf[KSTEPS];
-    u32x4 vf[KSTEPS];
+    // this wavefront's B operand: K^T (score role) or V^T (grad role); column = key, contraction over head dims
+    u32x4 of[KSTEPS];
+    {
+        const unsigned short* src = (grad_role ? v : k) + kv_head + (long long)kload * D + gh * 8;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-        kf[ks] = *reinterpret_cast<const u32x4*>(k + kv_head + (long long)kload * D + ks * 16 + gh * 8);
-        vf[ks] = *reinterpret_cast<const u32x4*>(v + kv_head + (long long)kload * D + ks * 16 + gh * 8);
+        for (int ks = 0; ks < KSTEPS; ++ks) of[ks] = *reinterpret_cast<const u32x4*>(src + ks * 16);
     }
     const float c2 = g.scale * kLog2e;
 
@@ -339,165 +361,224 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
     const int n_qt = q_tiles_all - q_first;
     const int n_iter = group * n_qt;
 
-    f32x16 dk_acc[CB];
-    f32x16 dv_acc[CB];
+    f32x16 acc[CB];  // dV^T (score role) or dK^T (grad role)
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            dk_acc[cb][i] = 0.0f;
-            dv_acc[cb][i] = 0.0f;
-        }
+        for (int i = 0; i < 16; ++i) acc[cb][i] = 0.0f;
 
     RTile qtile;
     RTile gtile;
     float row_val = 0.0f;  // threads 0..63: lse; threads 64..127: delta
     const int ld_off = RTile::global_offset(tid);
     const int st_off = RTile::lds_offset(tid);
-
-    // threads 0..63 fetch lse, 64..127 delta of the stage's queries (the upper half of the workgroup repeats
-    // them); the row load is issued before the tile loads so that waiting for it never waits for those
     const int row_slot = tid % QT;
     const bool row_is_delta = (tid / QT) & 1;
+    const bool row_thread = tid < 2 * QT;
+    const float neg_inv_scale = -1.0f / g.scale;
+
     auto load_stage = [&](int it) {
         const int h = kvh * group + it / n_qt;
         const int q0 = (q_first + it % n_qt) * QT;
         const long long q_head = ((long long)b * g.q_heads + h) * T * D;
-        const int t = min(q0 + row_slot, T - 1);
-        const float* row_src = row_is_delta ? delta + (long long)h * g.packs * T + (long long)b * T
-                                            : lse + b * lm.pack_stride + h * lm.head_stride;
-        row_val = row_src[t];
+        {   // every thread loads a row value (no branch); only the first 128 publish theirs
+            const int t = min(q0 + row_slot, T - 1);
+            const float* row_src = row_is_delta ? delta + (long long)h * g.packs * T + (long long)b * T
+                                                : lse + b * lm.pack_stride + h * lm.head_stride;
+            row_val = row_src[t];
+        }
         const __amdgpu_buffer_rsrc_t q_rsrc = make_head_rsrc(q + q_head, (long long)T * D * 2);
         const __amdgpu_buffer_rsrc_t g_rsrc = make_head_rsrc(d_out + q_head, (long long)T * D * 2);
         qtile.load(q_rsrc, ld_off, q0 * D * 2);
         gtile.load(g_rsrc, ld_off, q0 * D * 2);
     };
-    auto store_stage = [&](DkvLds<D>& st, int it) {
+    // Row values are published as accumulator start values: -lse / scale for the S chain (so that
+    // P = exp2(c * S) needs no subtraction) and -D for the dP chain.  -inf makes P = 0 for padded queries.
+    auto store_stage = [&](DkvSplitStage<D>& st, int it) {
         qtile.store(st.q, st_off);
         gtile.store(st.g, st_off);
-        const int q0 = (q_first + it % n_qt) * QT;
-        const bool live = q0 + row_slot < T;
-        if (tid < QT)
-            st.lse2[row_slot] = live ? row_val * kLog2e : __builtin_inff();  // exp2(s - inf) = 0 for padded queries
-        else if (tid < 2 * QT)
-            st.dl[row_slot] = live ? row_val : 0.0f;
+        if (row_thread) {
+            const int q0 = (q_first + it % n_qt) * QT;
+            const bool live = q0 + row_slot < T;
+            if (row_is_delta)
+                st.ndl[stage_slot(row_slot)] = live ? -row_val : 0.0f;
+            else
+                st.nls[stage_slot(row_slot)] = live ? row_val * neg_inv_scale : -__builtin_inff();
+        }
     };
 
-    // n_iter >= 1 always (the key tile's own queries)
     load_stage(0);
-    store_stage(lds[0], 0);
+    store_stage(lds.stage[0], 0);
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-        pin_loaded(kf[ks]);
-        pin_loaded(vf[ks]);
-    }
+    for (int ks = 0; ks < KSTEPS; ++ks) pin_loaded(of[ks]);
     __syncthreads();
 
-    const int r_off = row_perm(n) * QS + gh * 8;
-    const int t_off = transposed_read_offset(lane, QS);
+    // LDS addressing: one opaque per-lane byte offset per access pattern and stage, everything else is a
+    // compile-time constant that folds into the instruction's offset field.
+    constexpr int kStageBytes = (int)sizeof(DkvSplitStage<D>);
+    constexpr int kGOff = QT * QS;                    // elements from q to g
+    constexpr int kNlsBytes = 2 * QT * QS * 2;        // bytes from the stage start to nls
+    constexpr int kNdlBytes = kNlsBytes + QT * 4;
+    constexpr int kPBase = 3 * kStageBytes;           // bytes from the LDS start to p
+    constexpr int kPBufBytes = 4 * 2 * 2 * 64 * 16;
+    const int r_lane = (row_perm(n) * QS + gh * 8) * 2;
+    const int t_lane = transposed_read_offset(lane, QS) * 2;
+    const int v_lane = gh * 32;
+    const int p_lane = kPBase + kblock * (2 * 2 * 64 * 16) + lane * 16;
+    auto opaque = [](int x) {
+        asm volatile("" : "+v"(x));
+        return x;
+    };
+    auto tile_at = [&](int byte_off) { return reinterpret_cast<const unsigned short*>(dkv_smem + byte_off); };
 
-    // P and dS of one 32-query block from its S and dP tiles (this lane: one key, 16 queries), rounded and
-    // packed as the B operands of the dV / dK products.  MASKED is only instantiated for stages that touch
-    // the causal diagonal or the end of the sequence, so the common case carries no compare / select.
-    auto softmax_backward = [&](auto masked_tag, const f32x16& s, const f32x16& dp, const DkvLds<D>& st, int qb, int q0b,
-                                u32x4 (&pf)[2], u32x4 (&dsf)[2]) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
-        // lse and delta of the 16 queries this lane holds: rows 16*run + 8*gh + sigma(e), e = 0..7 (see mfma_tile.h)
-        float l2[16];
-        float dl[16];
+    // the 16 per-lane row values of a 32-query block, in register order
+    auto row_values = [&](int arr_off, int blk, f32x16& out) {
+        const float* arr = reinterpret_cast<const float*>(dkv_smem + arr_off);
 #pragma unroll
-        for (int run = 0; run < 2; ++run) {
-            float lrow[8];
-            float drow[8];
-#pragma unroll
-            for (int part = 0; part < 2; ++part) {
-                const int base = qb * 32 + run * 16 + gh * 8 + part * 4;
-                const float4 a = *reinterpret_cast<const float4*>(&st.lse2[base]);
-                const float4 d4 = *reinterpret_cast<const float4*>(&st.dl[base]);
-                lrow[part * 4] = a.x; lrow[part * 4 + 1] = a.y; lrow[part * 4 + 2] = a.z; lrow[part * 4 + 3] = a.w;
-                drow[part * 4] = d4.x; drow[part * 4 + 1] = d4.y; drow[part * 4 + 2] = d4.z; drow[part * 4 + 3] = d4.w;
-            }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                l2[run * 8 + e] = lrow[(e & 3) * 2 + (e >> 2)];
-                dl[run * 8 + e] = drow[(e & 3) * 2 + (e >> 2)];
-            }
-        }
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float p2[2];
-                float ds2[2];
-#pragma unroll
-                for (int w = 0; w < 2; ++w) {
-                    const int i = half * 8 + 2 * e + w;
-                    float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -l2[i]));
-                    if (MASKED) {
-                        const int query = q0b + perm_row_of_reg(i, gh);
-                        if ((CAUSAL && key > query) || key_dead) p = 0.0f;
-                    }
-                    p2[w] = p;
-                    ds2[w] = p * (dp[i] - dl[i]);
-                }
-                pf[half][e] = E::pack2(p2[0], p2[1]);
-                dsf[half][e] = E::pack2(ds2[0], ds2[1]);
-            }
+        for (int part = 0; part < 4; ++part) {
+            const float4 a = *reinterpret_cast<const float4*>(&arr[blk * 32 + (part >> 1) * 16 + (part & 1) * 4]);
+            out[part * 4 + 0] = a.x;
+            out[part * 4 + 1] = a.y;
+            out[part * 4 + 2] = a.z;
+            out[part * 4 + 3] = a.w;
         }
     };
 
-    // One stage = NB 32-query blocks.  Blocks entirely above the diagonal are not skipped (a few per
-    // workgroup): they are masked to zero instead, which keeps the stage body free of branches.
-    auto process_stage = [&](auto masked_tag, const DkvLds<D>& st, int q0) {
-        constexpr int NB = QT / 32;
-        f32x16 s[2];
-        f32x16 dp[2];
-        u32x4 pf[2][2];
-        u32x4 dsf[2][2];
-        auto scores = [&](int blk) {  // S and dP of block blk
+    // Operand fetches run one phase ahead of the matrix chain that consumes them: the LDS round trip is
+    // then hidden behind the previous chain or the softmax arithmetic instead of stalling every instruction.
+    auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
+    auto read_rows = [&](const unsigned short* at, u32x4 (&frag)[KSTEPS]) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                s[blk & 1][i] = 0.0f;
-                dp[blk & 1][i] = 0.0f;
-            }
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-                s[blk & 1] = E::mfma(lds_read128(&st.q[blk * 32 * QS + r_off + ks * 16]), kf[ks], s[blk & 1]);
-                dp[blk & 1] = E::mfma(lds_read128(&st.g[blk * 32 * QS + r_off + ks * 16]), vf[ks], dp[blk & 1]);
-            }
-        };
-        auto gradients = [&](int blk) {  // dV += dO^T P, dK += Q^T dS of block blk
-#pragma unroll
-            for (int c2i = 0; c2i < 2; ++c2i)
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    const u32x4 tg = lds_read_transposed(&st.g[t_off + (blk * 32 + c2i * 16) * QS + cb * 32], QS);
-                    dv_acc[cb] = E::mfma(tg, pf[blk & 1][c2i], dv_acc[cb]);
-                    const u32x4 tq = lds_read_transposed(&st.q[t_off + (blk * 32 + c2i * 16) * QS + cb * 32], QS);
-                    dk_acc[cb] = E::mfma(tq, dsf[blk & 1][c2i], dk_acc[cb]);
-                }
-        };
-#pragma unroll
-        for (int blk = 0; blk < NB; ++blk) {
-            scores(blk);
-            softmax_backward(masked_tag, s[blk & 1], dp[blk & 1], st, blk, q0 + blk * 32, pf[blk & 1], dsf[blk & 1]);
-            gradients(blk);
-        }
+        for (int ks = 0; ks < KSTEPS; ++ks) frag[ks] = lds_read128(at + ks * 16);
     };
-
-    // one trip of the stage loop: prefetch the next stage, work on this one, publish the next one
-    auto stage_trip = [&](auto masked_tag, int it) {
-        const bool more = it + 1 < n_iter;
-        if (more) load_stage(it + 1);
-        process_stage(masked_tag, lds[it & 1], (q_first + it % n_qt) * QT);
-        if (more) store_stage(lds[(it + 1) & 1], it + 1);
+    auto read_cols = [&](const unsigned short* at, u32x4 (&frag)[2][CB]) {  // token block of 32 at `at`
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) frag[half][cb] = lds_read_transposed(at + half * 16 * QS + cb * 32, QS);
+    };
+    // The next stage's global loads are issued just ahead of the last matrix chain of a trip (no LDS access
+    // follows them in the trip) and published to LDS behind it; then every wavefront meets at the barrier.
+    // Past the last stage the fetch repeats that stage into the (then unused) next buffer: no branch in a trip.
+    auto last_chain = [&](int it, auto&& chain) {
+        const int next = min(it + 1, n_iter - 1);
+        load_stage(next);
+        chain();
+        store_stage(lds.stage[(it + 1) % 3], next);
         __syncthreads();
     };
 
-    // Per query head of the group: the leading stages that touch this wavefront's causal diagonal (all stages if
-    // the key tile runs past the end of the sequence) take the masked code, the rest the unmasked code.  Two
-    // loops one after the other rather than a branch inside one loop, so the accumulators have one home.
-    {
+    // score role, trip `it`: P of both 32-query blocks of stage `it` -> LDS, dV^T += dO^T P
+    auto score_trip = [&](auto masked_tag, int it) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const int stage = it % 3;
+        const int q0 = (q_first + it % n_qt) * QT;
+        const unsigned short* rows = tile_at(opaque(stage * kStageBytes + r_lane));
+        const unsigned short* cols = tile_at(opaque(stage * kStageBytes + t_lane));
+        const int nls_off = opaque(stage * kStageBytes + kNlsBytes + v_lane);
+        u32x4* pout = reinterpret_cast<u32x4*>(dkv_smem + opaque(p_lane + (it & 1) * kPBufBytes));
+        // key - query of register i, block blk is mask_rel - (32 blk + row of register i in lane half 0): one
+        // per-lane value compared against compile-time constants; a key past the end masks everything
+        const int mask_rel = key_dead ? 0x7fffffff : (CAUSAL ? key - q0 - gh * 2 : -0x7fffffff);
+        u32x4 qrow[KSTEPS];
+        u32x4 gcol[2][CB];
+        f32x16 s;
+        read_rows(rows, qrow);
+        row_values(nls_off, 0, s);
+        fence();
+#pragma unroll
+        for (int blk = 0; blk < QT / 32; ++blk) {
+            // S chain (accumulator starts at -lse / scale); the dO^T operands of the dV chain are fetched meanwhile
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) s = E::mfma(qrow[ks], of[ks], s);
+            read_cols(cols + kGOff + blk * 32 * QS, gcol);
+            fence();
+            u32x4 pf[2];
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float p2[2];
+#pragma unroll
+                    for (int w = 0; w < 2; ++w) {
+                        const int i = half * 8 + 2 * e + w;
+                        float p = __builtin_amdgcn_exp2f(s[i] * c2);
+                        if (MASKED && mask_rel > blk * 32 + perm_row_of_reg(i, 0)) p = 0.0f;
+                        p2[w] = p;
+                    }
+                    pf[half][e] = E::pack2(p2[0], p2[1]);
+                }
+            pout[(blk * 2 + 0) * 64] = pf[0];
+            pout[(blk * 2 + 1) * 64] = pf[1];
+            auto dv_chain = [&] {
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) acc[cb] = E::mfma(gcol[half][cb], pf[half], acc[cb]);
+            };
+            if (blk + 1 < QT / 32) {  // next block's Q rows and row values: in flight during the dV chain
+                read_rows(rows + (blk + 1) * 32 * QS, qrow);
+                row_values(nls_off, blk + 1, s);
+                fence();
+                dv_chain();
+                fence();
+            } else {
+                fence();
+                last_chain(it, dv_chain);
+            }
+        }
+    };
+
+    // grad role, trip `it`: stage it - 1, dS = P o (dP - D), dK^T += Q^T dS
+    auto grad_trip = [&](int it) {
+        const int stage = (it - 1) % 3;
+        const unsigned short* rows = tile_at(opaque(stage * kStageBytes + r_lane));
+        const unsigned short* cols = tile_at(opaque(stage * kStageBytes + t_lane));
+        const int ndl_off = opaque(stage * kStageBytes + kNdlBytes + v_lane);
+        const u32x4* pin = reinterpret_cast<const u32x4*>(dkv_smem + opaque(p_lane + ((it - 1) & 1) * kPBufBytes));
+        u32x4 grow[KSTEPS];
+        u32x4 qcol[2][CB];
+        f32x16 dp;
+        read_rows(rows + kGOff, grow);
+        row_values(ndl_off, 0, dp);
+        fence();
+#pragma unroll
+        for (int blk = 0; blk < QT / 32; ++blk) {
+            // dP chain (accumulator starts at -D); P and the Q^T operands of the dK chain are fetched meanwhile
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) dp = E::mfma(grow[ks], of[ks], dp);
+            const u32x4 pf0 = pin[(blk * 2 + 0) * 64];
+            const u32x4 pf1 = pin[(blk * 2 + 1) * 64];
+            read_cols(cols + blk * 32 * QS, qcol);
+            fence();
+            u32x4 dsf[2];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                dsf[0][e] = E::pack2(E::lo(pf0[e]) * dp[2 * e], E::hi(pf0[e]) * dp[2 * e + 1]);
+                dsf[1][e] = E::pack2(E::lo(pf1[e]) * dp[8 + 2 * e], E::hi(pf1[e]) * dp[8 + 2 * e + 1]);
+            }
+            auto dk_chain = [&] {
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) acc[cb] = E::mfma(qcol[half][cb], dsf[half], acc[cb]);
+            };
+            if (blk + 1 < QT / 32) {
+                read_rows(rows + kGOff + (blk + 1) * 32 * QS, grow);
+                row_values(ndl_off, blk + 1, dp);
+                fence();
+                dk_chain();
+                fence();
+            } else {
+                fence();
+                last_chain(it, dk_chain);
+            }
+        }
+    };
+
+    // Trip i: the score wavefronts work on stage i, the grad wavefronts on stage i - 1 (trip 0 / trip n_iter
+    // are idle for the grad / score role).  Masked and unmasked score trips sit in loops of their own.
+    if (!grad_role) {
         int it = 0;
         for (int gi = 0; gi < group; ++gi) {
             const int head_end = (gi + 1) * n_qt;
@@ -506,25 +587,26 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 64 ? 2 : 1)) void dkdv_mfma_kern
                 masked_end = head_end;
             else if (CAUSAL)
                 masked_end = min(head_end, it + max(0, (k0w + 31 + QT - 1) / QT - q_first));
-            for (; it < masked_end; ++it) stage_trip(std::true_type{}, it);
-            for (; it < head_end; ++it) stage_trip(std::false_type{}, it);
+            for (; it < masked_end; ++it) score_trip(std::true_type{}, it);
+            for (; it < head_end; ++it) score_trip(std::false_type{}, it);
         }
+        __syncthreads();
+    } else {
+        last_chain(0, [] {});
+        for (int it = 1; it <= n_iter; ++it) grad_trip(it);
     }
 
     if (!key_dead) {
-        unsigned short* dkp = dk + kv_head + (long long)key * D;
-        unsigned short* dvp = dv + kv_head + (long long)key * D;
+        unsigned short* dst = (grad_role ? dk : dv) + kv_head + (long long)key * D;
+        const float out_scale = grad_role ? g.scale : 1.0f;
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                u32x2 wk, wv;
-                wk[0] = E::pack2(dk_acc[cb][a * 4 + 0] * g.scale, dk_acc[cb][a * 4 + 1] * g.scale);
-                wk[1] = E::pack2(dk_acc[cb][a * 4 + 2] * g.scale, dk_acc[cb][a * 4 + 3] * g.scale);
-                wv[0] = E::pack2(dv_acc[cb][a * 4 + 0], dv_acc[cb][a * 4 + 1]);
-                wv[1] = E::pack2(dv_acc[cb][a * 4 + 2], dv_acc[cb][a * 4 + 3]);
-                *reinterpret_cast<u32x2*>(dkp + cb * 32 + a * 8 + gh * 4) = wk;
-                *reinterpret_cast<u32x2*>(dvp + cb * 32 + a * 8 + gh * 4) = wv;
+                u32x2 w;
+                w[0] = E::pack2(acc[cb][a * 4 + 0] * out_scale, acc[cb][a * 4 + 1] * out_scale);
+                w[1] = E::pack2(acc[cb][a * 4 + 2] * out_scale, acc[cb][a * 4 + 3] * out_scale);
+                *reinterpret_cast<u32x2*>(dst + cb * 32 + a * 8 + gh * 4) = w;
             }
     }
 }
@@ -557,23 +639,23 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
         const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
         const int total = g.packs * g.kv_heads * k_tiles;
         const int grid = (total + 7) / 8 * 8;
-        const size_t smem = 2 * sizeof(DkvLds<D>);
+        const size_t smem = sizeof(DkvSplitLds<D>);
         static bool raised[2] = {false, false};  // one-time opt-in to more than 64 KiB of LDS per kernel
         const int which = g.causal ? 1 : 0;
         if (!raised[which]) {
-            const void* fn = g.causal ? reinterpret_cast<const void*>(dkdv_mfma_kernel<E, D, true>)
-                                      : reinterpret_cast<const void*>(dkdv_mfma_kernel<E, D, false>);
+            const void* fn = g.causal ? reinterpret_cast<const void*>(dkdv_split_kernel<E, D, true>)
+                                      : reinterpret_cast<const void*>(dkdv_split_kernel<E, D, false>);
             err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
             if (err != hipSuccess) return err;
             raised[which] = true;
         }
         KernelTimer timer("dkdv_mfma", stream);
         if (g.causal)
-            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, true>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp,
-                               lse, delta, dkp, dvp, lm, g, k_tiles, total);
+            hipLaunchKernelGGL((dkdv_split_kernel<E, D, true>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp,
+                               gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
         else
-            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, false>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp,
-                               lse, delta, dkp, dvp, lm, g, k_tiles, total);
+            hipLaunchKernelGGL((dkdv_split_kernel<E, D, false>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp,
+                               gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }

@@ -12,12 +12,13 @@
 //
 // To turn a D result straight into the B operand of the next product (contraction over its rows), the
 // rows of the first product are loaded in the order row_perm(): D row index m then carries matrix row
-// row_perm(m), chosen so that registers 0..7 of lane-half g hold rows 8g + {0,2,4,6,1,3,5,7} and registers
+// row_perm(m), chosen so that registers 0..7 of lane-half g hold rows 2g + {0,4,8,12,1,5,9,13} and registers
 // 8..15 the same rows + 16: the packing of a B operand for two consecutive k-steps whose contraction
-// index 8g + e stands for row 8g + sigma(e), sigma = {0,2,4,6,1,3,5,7}.  The matching A operand of the
-// second product is read with two transposing LDS reads that fetch the even and the odd rows of the
-// lane-half (lds_read_transposed); rows two apart is what keeps those reads free of bank conflicts with
-// the same 8-element row pad that suits the 128-bit row reads.
+// index (g, e) stands for row 2g + rho(e), rho = {0,4,8,12,1,5,9,13}.  The matching A operand of the
+// second product is read with two transposing LDS reads, each fetching four rows that lie four apart
+// (lds_read_transposed).  Rows four apart is what makes the 32 lanes that the LDS serves per cycle hit 64
+// different banks, with the 8-element row pad that also suits the 128-bit row reads (which only need the
+// 16 rows of a lane group to be 16 different rows) as well as with the XOR-swizzled unpadded layout.
 #ifndef SENTINEL_HIP_MFMA_TILE_H
 #define SENTINEL_HIP_MFMA_TILE_H
 
@@ -65,14 +66,14 @@ struct Fp16 {
     }
 };
 
-// Matrix row carried by D row index m = 8a + 4g + r (see the header comment): 16*(a/2) + 8g + 2r + a%2.
+// Matrix row carried by D row index m = 8a + 4g + r (see the header comment): 16*(a/2) + 4r + 2g + a%2.
 __device__ __forceinline__ int row_perm(int m) {
-    return (m & 16) | (((m >> 2) & 1) << 3) | ((m & 3) << 1) | ((m >> 3) & 1);
+    return (m & 16) | ((m & 3) << 2) | (((m >> 2) & 1) << 1) | ((m >> 3) & 1);
 }
 
 // Row (within a 32-row block) held by D register i of lane-half g when the rows were loaded through row_perm.
 __device__ __forceinline__ int perm_row_of_reg(int i, int g) {
-    return ((i >> 3) << 4) | (g << 3) | ((i & 3) << 1) | ((i >> 2) & 1);
+    return ((i >> 3) << 4) | ((i & 3) << 2) | (g << 1) | ((i >> 2) & 1);
 }
 
 // Plain D layout row of register i.
@@ -153,11 +154,11 @@ struct RowTile {
 // A operand whose contraction runs over the ROWS (tokens) of a row-major LDS tile: the transposed view
 // tile^T[col][token], read with ds_read_b64_tr_b16.  Within a 16-lane group that instruction returns to
 // lane i the 4 x 16-bit values {element i%4 of the 8 bytes addressed by lane 4j + i/4, j = 0..3}; with
-// lane i addressing tile[t0 + 2*(i/4)][c0 + 4*(i%4) ..] lane i therefore receives
-// tile[t0 + {0,2,4,6}][c0 + i]: the even tokens of one column; a second read one row further gives the
-// odd ones.  Together: contraction elements e = 0..7 of this lane-half = tokens t0 + sigma(e).
+// lane i addressing tile[t0 + 4*(i/4)][c0 + 4*(i%4) ..] lane i therefore receives
+// tile[t0 + {0,4,8,12}][c0 + i]: four tokens of one column; a second read one row further gives the
+// next four.  Together: contraction elements e = 0..7 of this lane-half = tokens t0 + rho(e).
 //   lane groups: lanes 0-15 -> columns c0..c0+15, lanes 16-31 -> c0+16..c0+31 (operand rows n = lane % 32),
-//   lanes 32-63 the same columns for the second half of the contraction (tokens + 8).
+//   lanes 32-63 the same columns for the second half of the contraction (tokens + 2).
 // ---------------------------------------------------------------------------------------------
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
@@ -165,14 +166,14 @@ __device__ __forceinline__ int transposed_read_offset(int lane, int stride) {
     const int i = lane & 15;
     const int column_block = (lane >> 4) & 1;
     const int gh = lane >> 5;
-    return (gh * 8 + 2 * (i >> 2)) * stride + column_block * 16 + 4 * (i & 3);
+    return (gh * 2 + 4 * (i >> 2)) * stride + column_block * 16 + 4 * (i & 3);
 }
 
 // tile_at = tile + transposed_read_offset + t0 * stride + c0
 __device__ __forceinline__ u32x4 lds_read_transposed(const unsigned short* tile_at, int stride) {
     typedef s16x4_t __attribute__((address_space(3))) * lds_ptr;
-    const s16x4_t even = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at));
-    const s16x4_t odd = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at + stride));
+    const s16x4_t even = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at));           // tokens rho(0..3)
+    const s16x4_t odd = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile_at + stride));  // tokens rho(4..7)
     const u32x2 a = __builtin_bit_cast(u32x2, even);
     const u32x2 b = __builtin_bit_cast(u32x2, odd);
     u32x4 r = {a[0], a[1], b[0], b[1]};
@@ -184,8 +185,8 @@ __device__ __forceinline__ u32x4 lds_read_transposed(const unsigned short* tile_
 // tile + 16 * (chunk index) in issue order, so the tile is unpadded; bank conflicts are avoided by an XOR
 // swizzle instead: the 16-byte chunk c of row r is kept at chunk position c ^ (r mod chunks_per_row),
 // which is applied on the global side (each lane fetches the chunk that belongs at its position).
-// Both operand read patterns stay conflict-free: 16 consecutive rows of one logical chunk hit 16 different
-// positions, and the transposed reads touch rows two apart whose chunk pairs fall on different positions.
+// Both operand read patterns stay conflict-free: 16 different rows (mod 16) of one logical chunk hit 16
+// different positions, and the four rows (four apart) times four chunks of a transposed read likewise.
 // ---------------------------------------------------------------------------------------------
 template <int ROWS, int D, int THREADS>
 struct DirectTile {
@@ -213,11 +214,11 @@ struct DirectTile {
     }
     // element offset of this lane's 128-bit operand read of row `row` (k-step 0): xor (ks << 4) selects k-step ks
     static __device__ __forceinline__ int row_read_base(int row, int gh) { return row * D + ((gh ^ (row & kMask)) << 3); }
-    // element offsets of this lane's two transposed reads (even / odd tokens) for token block 0, column block 0:
+    // element offsets of this lane's two transposed reads (tokens rho(0..3) / rho(4..7)) for token block 0, column block 0:
     // add t0 * D for the token block (t0 a multiple of 16), xor (cb << 5) for column block cb
     static __device__ __forceinline__ int transposed_read_base(int lane, int odd) {
         const int i = lane & 15;
-        const int r = (lane >> 5) * 8 + 2 * (i >> 2) + odd;
+        const int r = (lane >> 5) * 2 + 4 * (i >> 2) + odd;
         const int chunk = ((lane >> 4) & 1) * 2 + ((i & 3) >> 1);
         return r * D + ((chunk ^ (r & kMask)) << 3) + 4 * (i & 1);
     }
