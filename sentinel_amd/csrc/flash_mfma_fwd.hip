@@ -23,6 +23,11 @@ namespace {
 
 constexpr int kFwdThreads = 256;
 constexpr int kFwdQueryTile = 128;
+// instruction classes of __builtin_amdgcn_sched_group_barrier
+constexpr int kSchedMfma = 0x008;
+constexpr int kSchedDsRead = 0x100;
+constexpr int kOperandLead = 4;
+
 constexpr int kFwdKeyTile = 64;
 
 template <typename E, int D, bool CAUSAL>
@@ -118,17 +123,39 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
         // wavefront-uniform: the whole tile lies above this wavefront's diagonal
         const bool skip = CAUSAL && key0 > q0w + 31;
         if (!skip) {
+            // S^T chains with their K operands read kOperandLead instructions ahead; the V^T operands of the first
+            // half of the PV product are fetched behind them and land during the softmax arithmetic
             f32x16 s[2];
+            u32x4 kfrag[2][KSTEPS];
+            u32x4 vfrag[4][CB];
+#pragma unroll
+            for (int kbk = 0; kbk < 2; ++kbk)
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks) kfrag[kbk][ks] = lds_read128(&k_lds[buf][kbk * 32 * KS + k_off + ks * 16]);
 #pragma unroll
             for (int kbk = 0; kbk < 2; ++kbk) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) s[kbk][i] = 0.0f;
 #pragma unroll
-                for (int ks = 0; ks < KSTEPS; ++ks) {
-                    const u32x4 a = lds_read128(&k_lds[buf][kbk * 32 * KS + k_off + ks * 16]);
-                    s[kbk] = E::mfma(a, qf[ks], s[kbk]);
-                }
+                for (int ks = 0; ks < KSTEPS; ++ks) s[kbk] = E::mfma(kfrag[kbk][ks], qf[ks], s[kbk]);
             }
+#pragma unroll
+            for (int c4 = 0; c4 < 2; ++c4)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+                    vfrag[c4][cb] = lds_read_transposed(&v_lds[buf][v_off + c4 * 16 * VS + cb * 32], VS);
+            __builtin_amdgcn_sched_group_barrier(kSchedDsRead, kOperandLead, 0);
+#pragma unroll
+            for (int i = 0; i < 2 * KSTEPS - kOperandLead; ++i) {
+                __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < kOperandLead; ++i) {
+                __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 4 * CB / kOperandLead, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
 
             const bool need_mask = (CAUSAL && key0 + KT - 1 > q0w) || (!CAUSAL && key0 + KT > T);
             if (need_mask) {
@@ -178,14 +205,24 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             }
             l_run += psum;
 
+            __builtin_amdgcn_sched_barrier(0);
+            // PV: the first half runs on the operands fetched above while the second half's are read
 #pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4) {
+            for (int c4 = 2; c4 < 4; ++c4)
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    const u32x4 a = lds_read_transposed(&v_lds[buf][v_off + c4 * 16 * VS + cb * 32], VS);
-                    acc[cb] = E::mfma(a, pf[c4], acc[cb]);
-                }
+                for (int cb = 0; cb < CB; ++cb)
+                    vfrag[c4][cb] = lds_read_transposed(&v_lds[buf][v_off + c4 * 16 * VS + cb * 32], VS);
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) acc[cb] = E::mfma(vfrag[c4][cb], pf[c4], acc[cb]);
+#pragma unroll
+            for (int i = 0; i < 2 * CB; ++i) {
+                __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 2, 0);
             }
+            __builtin_amdgcn_sched_group_barrier(kSchedMfma, 2 * CB, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
 
         if (more) {
