@@ -147,6 +147,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[cb][i] = 0.0f;
 
+    const int mask_base = (CAUSAL ? min(qrow, T - 1) : T - 1) - 2 * gh;  // last live key of this lane's query, minus the lane half's row offset
     const int k_off = Tile::row_read_base(row_perm(n), gh);
     const int t_even = Tile::transposed_read_base(lane, 0);
     const int t_odd = Tile::transposed_read_base(lane, 1);
@@ -200,11 +201,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -lse2));
-                    if (MASKED) {
-                        const int key = key0 + kbk * 32 + perm_row_of_reg(i, gh);
-                        const bool dead = CAUSAL ? key > qrow : key >= T;
-                        if (dead) p[i] = 0.0f;
-                    }
+                    // dead iff key0 + 32 kbk + (row of register i in lane half 0) + 2 gh > last live key
+                    if (MASKED && perm_row_of_reg(i, 0) > mask_base - key0 - kbk * 32) p[i] = 0.0f;
                 }
                 u32x4 dsf[2];
 #pragma unroll
@@ -219,7 +217,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 #pragma unroll
                     for (int cb = 0; cb < CB; ++cb) acc[cb] = E::mfma(kt_frag[half][cb], dsf[half], acc[cb]);
                 }
-                if (!MASKED) {
+                {
                     // S chain with its operand reads kOperandLead ahead, then the dP chain overlapped with exp(S) and
                     // the transposed reads of the dQ operands, then the rest of the arithmetic, then the dQ chain
                     __builtin_amdgcn_sched_group_barrier(kSchedDsRead, kOperandLead, 0);
@@ -305,6 +303,254 @@ struct DkvSplitLds {
 // so four 128-bit reads fill the 16 per-lane values in register order.
 __device__ __forceinline__ int stage_slot(int r) {
     return (r & ~15) | (((r >> 1) & 1) << 3) | ((r & 1) << 2) | ((r >> 2) & 3);
+}
+
+// ------------------------------------------------------------------------------------------------
+// dK, dV for head dims up to 64: one wavefront per 32-key block holds K, V (as B operands) and both
+// accumulators and still leaves room for two wavefronts per SIMD, so the work is not split over roles.
+// ------------------------------------------------------------------------------------------------
+template <int D>
+struct DkvLds {
+    static constexpr int QT = kDkvQueryTile;
+    static constexpr int kPad = 8;  // row pad (elements): conflict-free for the 128-bit row reads and the transposed reads
+    static constexpr int QS = D + kPad;
+    unsigned short q[QT * QS];
+    unsigned short g[QT * QS];
+    float lse2[QT];
+    float dl[QT];
+};
+
+template <typename E, int D, bool CAUSAL>
+__global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
+    const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
+    const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
+    unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
+    int total_tiles) {
+    constexpr int QT = kDkvQueryTile;
+    typedef RowTile<QT, D, kBwdThreads, DkvLds<D>::kPad> RTile;
+    constexpr int QS = RTile::kStride;
+    static_assert(QS == DkvLds<D>::QS, "LDS layout mismatch");
+    constexpr int KSTEPS = D / 16;
+    constexpr int CB = D / 32;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char dkv_smem[];
+    DkvLds<D>* lds = reinterpret_cast<DkvLds<D>*>(dkv_smem);  // two stages
+
+    const int per_xcd = (int)gridDim.x / 8;
+    const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
+    if (tile_id >= total_tiles) return;
+    const int bkv = tile_id / k_tiles;
+    const int ktile = tile_id % k_tiles;  // under the causal mask the first key tiles see the most queries
+    const int b = bkv / g.kv_heads;
+    const int kvh = bkv % g.kv_heads;
+    const int group = g.q_heads / g.kv_heads;
+    const int T = g.seq_len;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);  // wavefront-uniform by construction; tell the compiler
+    const int lane = tid % 64;
+    const int n = lane % 32;
+    const int gh = lane / 32;
+
+    const long long kv_head = ((long long)b * g.kv_heads + kvh) * T * D;
+    const int k0w = ktile * kDkvKeyTile + wave * 32;
+    const int key = k0w + n;
+    const int kload = key < T ? key : T - 1;
+    const bool key_dead = key >= T;
+
+    // K^T and V^T as B operands: column = key, contraction over head dims
+    u32x4 kf[KSTEPS];
+    u32x4 vf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        kf[ks] = *reinterpret_cast<const u32x4*>(k + kv_head + (long long)kload * D + ks * 16 + gh * 8);
+        vf[ks] = *reinterpret_cast<const u32x4*>(v + kv_head + (long long)kload * D + ks * 16 + gh * 8);
+    }
+    const float c2 = g.scale * kLog2e;
+
+    const int q_tiles_all = (T + QT - 1) / QT;
+    const int q_first = CAUSAL ? (ktile * kDkvKeyTile) / QT : 0;
+    const int n_qt = q_tiles_all - q_first;
+    const int n_iter = group * n_qt;
+
+    f32x16 dk_acc[CB];
+    f32x16 dv_acc[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            dk_acc[cb][i] = 0.0f;
+            dv_acc[cb][i] = 0.0f;
+        }
+
+    RTile qtile;
+    RTile gtile;
+    float row_val = 0.0f;  // threads 0..63: lse; threads 64..127: delta
+    const int ld_off = RTile::global_offset(tid);
+    const int st_off = RTile::lds_offset(tid);
+
+    // threads 0..63 fetch lse, 64..127 delta of the stage's queries (the upper half of the workgroup repeats
+    // them); the row load is issued before the tile loads so that waiting for it never waits for those
+    const int row_slot = tid % QT;
+    const bool row_is_delta = (tid / QT) & 1;
+    auto load_stage = [&](int it) {
+        const int h = kvh * group + it / n_qt;
+        const int q0 = (q_first + it % n_qt) * QT;
+        const long long q_head = ((long long)b * g.q_heads + h) * T * D;
+        const int t = min(q0 + row_slot, T - 1);
+        const float* row_src = row_is_delta ? delta + (long long)h * g.packs * T + (long long)b * T
+                                            : lse + b * lm.pack_stride + h * lm.head_stride;
+        row_val = row_src[t];
+        const __amdgpu_buffer_rsrc_t q_rsrc = make_head_rsrc(q + q_head, (long long)T * D * 2);
+        const __amdgpu_buffer_rsrc_t g_rsrc = make_head_rsrc(d_out + q_head, (long long)T * D * 2);
+        qtile.load(q_rsrc, ld_off, q0 * D * 2);
+        gtile.load(g_rsrc, ld_off, q0 * D * 2);
+    };
+    auto store_stage = [&](DkvLds<D>& st, int it) {
+        qtile.store(st.q, st_off);
+        gtile.store(st.g, st_off);
+        const int q0 = (q_first + it % n_qt) * QT;
+        const bool live = q0 + row_slot < T;
+        if (tid < QT)
+            st.lse2[stage_slot(row_slot)] = live ? row_val * kLog2e : __builtin_inff();  // exp2(s - inf) = 0 for padded queries
+        else if (tid < 2 * QT)
+            st.dl[stage_slot(row_slot)] = live ? row_val : 0.0f;
+    };
+
+    // n_iter >= 1 always (the key tile's own queries)
+    load_stage(0);
+    store_stage(lds[0], 0);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        pin_loaded(kf[ks]);
+        pin_loaded(vf[ks]);
+    }
+    __syncthreads();
+
+    const int r_off = row_perm(n) * QS + gh * 8;
+    const int t_off = transposed_read_offset(lane, QS);
+
+    // P and dS of one 32-query block from its S and dP tiles (this lane: one key, 16 queries), rounded and
+    // packed as the B operands of the dV / dK products.  MASKED is only instantiated for stages that touch
+    // the causal diagonal or the end of the sequence, so the common case carries no compare / select.
+    auto softmax_backward = [&](auto masked_tag, const f32x16& s, const f32x16& dp, const DkvLds<D>& st, int qb, int q0b,
+                                u32x4 (&pf)[2], u32x4 (&dsf)[2]) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        // lse and delta of the 16 queries this lane holds, in register order (the arrays are kept in that order)
+        float l2[16];
+        float dl[16];
+#pragma unroll
+        for (int part = 0; part < 4; ++part) {
+            const int base = qb * 32 + (part >> 1) * 16 + gh * 8 + (part & 1) * 4;
+            const float4 a = *reinterpret_cast<const float4*>(&st.lse2[base]);
+            const float4 d4 = *reinterpret_cast<const float4*>(&st.dl[base]);
+            l2[part * 4] = a.x; l2[part * 4 + 1] = a.y; l2[part * 4 + 2] = a.z; l2[part * 4 + 3] = a.w;
+            dl[part * 4] = d4.x; dl[part * 4 + 1] = d4.y; dl[part * 4 + 2] = d4.z; dl[part * 4 + 3] = d4.w;
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float p2[2];
+                float ds2[2];
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    const int i = half * 8 + 2 * e + w;
+                    float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -l2[i]));
+                    if (MASKED) {
+                        const int query = q0b + perm_row_of_reg(i, gh);
+                        if ((CAUSAL && key > query) || key_dead) p = 0.0f;
+                    }
+                    p2[w] = p;
+                    ds2[w] = p * (dp[i] - dl[i]);
+                }
+                pf[half][e] = E::pack2(p2[0], p2[1]);
+                dsf[half][e] = E::pack2(ds2[0], ds2[1]);
+            }
+        }
+    };
+
+    // One stage = NB 32-query blocks.  Blocks entirely above the diagonal are not skipped (a few per
+    // workgroup): they are masked to zero instead, which keeps the stage body free of branches.
+    auto process_stage = [&](auto masked_tag, const DkvLds<D>& st, int q0) {
+        constexpr int NB = QT / 32;
+        f32x16 s[2];
+        f32x16 dp[2];
+        u32x4 pf[2][2];
+        u32x4 dsf[2][2];
+        auto scores = [&](int blk) {  // S and dP of block blk
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                s[blk & 1][i] = 0.0f;
+                dp[blk & 1][i] = 0.0f;
+            }
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                s[blk & 1] = E::mfma(lds_read128(&st.q[blk * 32 * QS + r_off + ks * 16]), kf[ks], s[blk & 1]);
+                dp[blk & 1] = E::mfma(lds_read128(&st.g[blk * 32 * QS + r_off + ks * 16]), vf[ks], dp[blk & 1]);
+            }
+        };
+        auto gradients = [&](int blk) {  // dV += dO^T P, dK += Q^T dS of block blk
+#pragma unroll
+            for (int c2i = 0; c2i < 2; ++c2i)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const u32x4 tg = lds_read_transposed(&st.g[t_off + (blk * 32 + c2i * 16) * QS + cb * 32], QS);
+                    dv_acc[cb] = E::mfma(tg, pf[blk & 1][c2i], dv_acc[cb]);
+                    const u32x4 tq = lds_read_transposed(&st.q[t_off + (blk * 32 + c2i * 16) * QS + cb * 32], QS);
+                    dk_acc[cb] = E::mfma(tq, dsf[blk & 1][c2i], dk_acc[cb]);
+                }
+        };
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk) {
+            scores(blk);
+            softmax_backward(masked_tag, s[blk & 1], dp[blk & 1], st, blk, q0 + blk * 32, pf[blk & 1], dsf[blk & 1]);
+            gradients(blk);
+        }
+    };
+
+    // one trip of the stage loop: prefetch the next stage, work on this one, publish the next one
+    auto stage_trip = [&](auto masked_tag, int it) {
+        const bool more = it + 1 < n_iter;
+        if (more) load_stage(it + 1);
+        process_stage(masked_tag, lds[it & 1], (q_first + it % n_qt) * QT);
+        if (more) store_stage(lds[(it + 1) & 1], it + 1);
+        __syncthreads();
+    };
+
+    // Per query head of the group: the leading stages that touch this wavefront's causal diagonal (all stages if
+    // the key tile runs past the end of the sequence) take the masked code, the rest the unmasked code.  Two
+    // loops one after the other rather than a branch inside one loop, so the accumulators have one home.
+    {
+        int it = 0;
+        for (int gi = 0; gi < group; ++gi) {
+            const int head_end = (gi + 1) * n_qt;
+            int masked_end = it;
+            if (k0w + 31 >= T)
+                masked_end = head_end;
+            else if (CAUSAL)
+                masked_end = min(head_end, it + max(0, (k0w + 31 + QT - 1) / QT - q_first));
+            for (; it < masked_end; ++it) stage_trip(std::true_type{}, it);
+            for (; it < head_end; ++it) stage_trip(std::false_type{}, it);
+        }
+    }
+
+    if (!key_dead) {
+        unsigned short* dkp = dk + kv_head + (long long)key * D;
+        unsigned short* dvp = dv + kv_head + (long long)key * D;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                u32x2 wk, wv;
+                wk[0] = E::pack2(dk_acc[cb][a * 4 + 0] * g.scale, dk_acc[cb][a * 4 + 1] * g.scale);
+                wk[1] = E::pack2(dk_acc[cb][a * 4 + 2] * g.scale, dk_acc[cb][a * 4 + 3] * g.scale);
+                wv[0] = E::pack2(dv_acc[cb][a * 4 + 0], dv_acc[cb][a * 4 + 1]);
+                wv[1] = E::pack2(dv_acc[cb][a * 4 + 2], dv_acc[cb][a * 4 + 3]);
+                *reinterpret_cast<u32x2*>(dkp + cb * 32 + a * 8 + gh * 4) = wk;
+                *reinterpret_cast<u32x2*>(dvp + cb * 32 + a * 8 + gh * 4) = wv;
+            }
+    }
 }
 
 template <typename E, int D, bool CAUSAL>
@@ -635,7 +881,21 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
     if (err != hipSuccess) return err;
 
     // dK, dV
-    {
+    if constexpr (D <= 64) {
+        const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
+        const int total = g.packs * g.kv_heads * k_tiles;
+        const int grid = (total + 7) / 8 * 8;
+        const size_t smem = 2 * sizeof(DkvLds<D>);
+        KernelTimer timer("dkdv_mfma", stream);
+        if (g.causal)
+            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, true>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp,
+                               lse, delta, dkp, dvp, lm, g, k_tiles, total);
+        else
+            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, false>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp,
+                               lse, delta, dkp, dvp, lm, g, k_tiles, total);
+        err = hipGetLastError();
+        if (err != hipSuccess) return err;
+    } else {
         const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
         const int total = g.packs * g.kv_heads * k_tiles;
         const int grid = (total + 7) / 8 * 8;
