@@ -86,6 +86,18 @@ class Workload:
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps * 1e3  # ms per call
 
+    def event_times(self, fn, steps):
+        """Per-call durations (ms) from events on the launch stream (torch's current stream)."""
+        torch = self.torch
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        for i in range(steps):
+            starts[i].record()
+            fn()
+            stops[i].record()
+        torch.cuda.synchronize()
+        return sorted(a.elapsed_time(b) for a, b in zip(starts, stops))
+
     def kernel_times(self, steps):
         """Average duration of each kernel over `steps` timed steps (hipEvents on the launch stream)."""
         self.fa.set_kernel_timing(True)
@@ -97,8 +109,21 @@ class Workload:
         return {k: total / max(n, 1) for k, (total, n) in times.items()}
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(name, heads_sample):
-    """The CPU oracle (a restatement of the reference's OpenMP attention) timed on a bounded sample."""
+    """The CPU oracle (a restatement of the reference's OpenMP attention) timed on a bounded sample, in the two
+    ways the reference runs it: one sequence at a time with the matrix products OpenMP-parallel inside
+    ("single-call"), and one thread per sequence of the batch with serial products ("train-loop")."""
     import numpy as np
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib
@@ -106,33 +131,68 @@ def cpu_baseline(name, heads_sample):
     group = hq // hkv
     heads_sample = max(group, min(hq, heads_sample) // group * group)
     kv_sample = heads_sample // group
-    rng = np.random.default_rng(0x5E17)
-    q = (sigma * rng.standard_normal((heads_sample * d, t))).astype(np.float32)
-    k = (sigma * rng.standard_normal((kv_sample * d, t))).astype(np.float32)
-    v = rng.standard_normal((kv_sample * d, t)).astype(np.float32)
-    g = rng.standard_normal((heads_sample * d, t)).astype(np.float32)
     threads = oracle_lib.oracle().sentinel_oracle_max_threads()
+    rng = np.random.default_rng(0x5E17)
+
+    def draw(packs):
+        q = (sigma * rng.standard_normal((heads_sample * d, packs * t))).astype(np.float32)
+        k = (sigma * rng.standard_normal((kv_sample * d, packs * t))).astype(np.float32)
+        v = rng.standard_normal((kv_sample * d, packs * t)).astype(np.float32)
+        g = rng.standard_normal((heads_sample * d, packs * t)).astype(np.float32)
+        return q, k, v, g
+
+    # single-call mode: 1 sequence x heads_sample heads
+    q, k, v, g = draw(1)
     t0 = time.perf_counter()
     oracle_lib.oracle_attention(q, k, v, g, q_heads=heads_sample, kv_heads=kv_sample, head_dim=d, seq_len=t)
     dt = time.perf_counter() - t0
     flops = 7.0 * heads_sample * t * t * d
+    # train-loop mode: the b sequences of the batch in parallel, one K/V head group each
+    heads_loop = group
+    heads_sample, kv_sample = heads_loop, heads_loop // group
+    q, k, v, g = draw(b)
+    t1 = time.perf_counter()
+    oracle_lib.oracle_attention(q, k, v, g, q_heads=heads_loop, kv_heads=kv_sample, head_dim=d, seq_len=t, pack_count=b,
+                                pack_parallel=True)
+    dt_loop = time.perf_counter() - t1
+    flops_loop = 7.0 * b * heads_loop * t * t * d
     return {
         "value": flops / dt / 1e12,
         "unit": "TFLOP/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"1 sequence x {heads_sample} of {b * hq} (batch, head) pairs of {name}, fp32, forward+backward, "
-                  f"{dt:.1f} s; gemm/softmax OpenMP-parallel as in the reference's single-call mode; "
-                  "same causal FLOP count although the CPU path multiplies the full T x T",
+        "cpu": cpu_model(),
+        "sample": f"single-call mode: 1 sequence x {flops / (7.0 * t * t * d):.0f} of {b * hq} (batch, head) pairs of {name}, fp32, "
+                  f"forward+backward, {dt:.1f} s, gemm/softmax OpenMP-parallel inside; same causal FLOP count although the "
+                  "CPU path multiplies the full T x T",
         "seconds": dt,
+        "train_loop_mode": {"value": flops_loop / dt_loop / 1e12, "unit": "TFLOP/s", "cores": min(threads, b),
+                            "seconds": dt_loop,
+                            "sample": f"{b} sequences in parallel (one thread each, serial products) x {heads_loop} heads"},
     }
+
+
+def rocminfo_gpu_clock_ghz():
+    """Max Clock Freq. of the first gfx agent as printed by rocminfo (GHz), 0.0 if it cannot be read."""
+    import re
+    import subprocess
+    try:
+        text = subprocess.run(["/opt/rocm/bin/rocminfo"], capture_output=True, text=True, timeout=30).stdout
+    except (OSError, subprocess.SubprocessError):
+        return 0.0
+    for block in text.split("*******")[1:]:
+        if re.search(r"Name:\s+gfx", block):
+            m = re.search(r"Max Clock Freq\. \(MHz\):\s+(\d+)", block)
+            if m:
+                return int(m.group(1)) / 1e3
+    return 0.0
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="nstar", choices=sorted(CONFIGS))
     ap.add_argument("--cpu-heads", type=int, default=8, help="(batch, head) pairs in the CPU baseline sample; 0 = skip")
     ap.add_argument("--no-configs", action="store_true", help="skip the brief timing of the other configurations")
@@ -152,11 +212,23 @@ def main():
         sys.exit(3)
     sentinel_amd.load_library()
 
+    props = torch.cuda.get_device_properties(0)
+    cus = int(props.multi_processor_count)
+    clock_ghz = float(getattr(props, "clock_rate", 0)) / 1e6  # kHz -> GHz
+    if clock_ghz <= 0.0:  # not filled in by this torch build: ask rocminfo for the GPU agent's maximum clock
+        clock_ghz = rocminfo_gpu_clock_ghz()
+    device = {"name": props.name, "compute_units": cus, "max_clock_ghz": clock_ghz,
+              # dense bf16 / fp16 MFMA: 4096 FLOP per clock per CU; the fraction below uses the published figure
+              "mfma_peak_from_device_tflops": cus * 4096 * clock_ghz / 1e3}
+
     w = Workload(torch, args.config)
     ms_step = w.timed(w.step, args.steps, args.warmup)
-    ms_fwd = w.timed(w.forward, max(args.steps // 2, 1), 1)
-    ms_bwd = w.timed(w.backward, max(args.steps // 2, 1), 1)
-    kernels = w.kernel_times(args.steps)
+    ev_step = w.event_times(w.step, args.steps)
+    ev_fwd = w.event_times(w.forward, args.steps)
+    ev_bwd = w.event_times(w.backward, args.steps)
+    ms_fwd = ev_fwd[len(ev_fwd) // 2]
+    ms_bwd = ev_bwd[len(ev_bwd) // 2]
+    kernels = w.kernel_times(min(args.steps, 20))
     if args.copy_calibration:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB read, 1 GiB written per launch
         dst = torch.empty_like(src)
@@ -196,6 +268,12 @@ def main():
         "bwd_ms": ms_bwd,
         "fwd_tflops": 2.0 * w.unit_flops / (ms_fwd * 1e-3) / 1e12,
         "bwd_tflops": 5.0 * w.unit_flops / (ms_bwd * 1e-3) / 1e12,
+        "step_ms_median_min": [ev_step[len(ev_step) // 2], ev_step[0]],
+        "fwd_ms_median_min": [ms_fwd, ev_fwd[0]],
+        "bwd_ms_median_min": [ms_bwd, ev_bwd[0]],
+        "timing": "value: wall clock over the timed steps; *_median_min: per-call events on the launch stream; "
+                  "buffers allocated once, L2 not flushed",
+        "device": device,
         "kernels_ms": kernels,
         "roofline": roofline,
     }
