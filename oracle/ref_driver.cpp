@@ -166,3 +166,35 @@ extern "C" int sentinel_ref_softmax_columns(const float* logits, float* out, int
         return -2;
     }
 }
+
+// The reference's own RotaryEmbedding (Layers/RotaryEmbedding.cpp): tables and the in-place rotation of a
+// rows x columns matrix (column = position; the host layer has no offset / segment rule).
+extern "C" int sentinel_ref_rope_tables(int headDim, int positions, float base, float* cosTable, float* sinTable) {
+    try {
+        const RotaryEmbedding rope(headDim, positions, base);
+        std::copy(rope.cosTable.begin(), rope.cosTable.end(), cosTable);
+        std::copy(rope.sinTable.begin(), rope.sinTable.end(), sinTable);
+        return 0;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}
+
+extern "C" int sentinel_ref_rope_rotate(float* tensor, int heads, int headDim, int columns, int positions, float base,
+                                        int inverse) {
+    try {
+        const RotaryEmbedding rope(headDim, positions, base);
+        Matrix m(static_cast<size_t>(heads) * headDim, static_cast<size_t>(columns), 0.0f);
+        for (size_t r = 0; r < m.rows; ++r)
+            for (size_t c = 0; c < m.cols; ++c) m.at(r, c) = tensor[r * m.cols + c];
+        if (inverse)
+            rope.rotateInverseInPlace(m, heads);
+        else
+            rope.rotateInPlace(m, heads);
+        for (size_t r = 0; r < m.rows; ++r)
+            for (size_t c = 0; c < m.cols; ++c) tensor[r * m.cols + c] = m.at(r, c);
+        return 0;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}

@@ -331,6 +331,55 @@ extern "C" int sentinel_oracle_softmax_columns(const float* logits, float* out, 
     return 0;
 }
 
+// Layers/RotaryEmbedding.cpp:8-29
+extern "C" int sentinel_oracle_rope_tables(int headDim, int positions, float base, float* cosTable, float* sinTable) {
+    if (headDim <= 0 || headDim % 2 != 0 || positions <= 0 || !(base > 0.0f) || !cosTable || !sinTable) return -1;
+    const int pairCount = headDim / 2;
+    for (int position = 0; position < positions; ++position) {
+        for (int pairIndex = 0; pairIndex < pairCount; ++pairIndex) {
+            const float exponent = -2.0f * static_cast<float>(pairIndex) / static_cast<float>(headDim);
+            const float angle = static_cast<float>(position) * std::pow(base, exponent);
+            const size_t tableIndex = static_cast<size_t>(position) * pairCount + pairIndex;
+            cosTable[tableIndex] = std::cos(angle);
+            sinTable[tableIndex] = std::sin(angle);
+        }
+    }
+    return 0;
+}
+
+// Layers/RotaryEmbedding.cpp:39-81 with the device position rule of Cuda/CudaOps.cu:362-402
+extern "C" int sentinel_oracle_rope_rotate(float* tensor, int heads, int headDim, int strideColumns, int colStart,
+                                           int columns, int positionOffset, int segmentLength, const float* cosTable,
+                                           const float* sinTable, int tablePositions, int inverse) {
+    if (!tensor || !cosTable || !sinTable || heads <= 0 || headDim <= 0 || headDim % 2 != 0) return -1;
+    if (columns < 0 || colStart < 0 || colStart + columns > strideColumns) return -1;
+    if (positionOffset < 0 || segmentLength < 0) return -1;
+    if (segmentLength > 0 ? segmentLength > tablePositions : positionOffset + columns > tablePositions) return -1;
+    const int pairCount = headDim / 2;
+    for (int headIndex = 0; headIndex < heads; ++headIndex) {
+        const size_t rowOffset = static_cast<size_t>(headIndex) * headDim;
+        for (int column = 0; column < columns; ++column) {
+            const int position = segmentLength > 0 ? column % segmentLength : positionOffset + column;
+            for (int pairIndex = 0; pairIndex < pairCount; ++pairIndex) {
+                float* even = tensor + (rowOffset + 2 * pairIndex) * strideColumns + colStart + column;
+                float* odd = even + strideColumns;
+                const float cosValue = cosTable[static_cast<size_t>(position) * pairCount + pairIndex];
+                const float sinValue = sinTable[static_cast<size_t>(position) * pairCount + pairIndex];
+                const float evenValue = *even;
+                const float oddValue = *odd;
+                if (!inverse) {
+                    *even = evenValue * cosValue - oddValue * sinValue;
+                    *odd = evenValue * sinValue + oddValue * cosValue;
+                } else {
+                    *even = evenValue * cosValue + oddValue * sinValue;
+                    *odd = -evenValue * sinValue + oddValue * cosValue;
+                }
+            }
+        }
+    }
+    return 0;
+}
+
 extern "C" int sentinel_oracle_max_threads(void) {
 #if defined(_OPENMP)
     return omp_get_max_threads();

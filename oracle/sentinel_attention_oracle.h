@@ -56,6 +56,25 @@ int sentinel_oracle_gemm(const float* a, int aRows, int aCols, const float* b, i
 /* column softmax (Activations/Softmax.cpp:10-44); rows x cols, row-major */
 int sentinel_oracle_softmax_columns(const float* logits, float* out, int rows, int cols);
 
+/*
+ * Rotary position embedding, the step on either side of the attention core.
+ *
+ * sentinel_oracle_rope_tables: cos / sin tables [positions][headDim / 2] exactly as the
+ * reference builds them (Layers/RotaryEmbedding.cpp:8-29: float pow, cos, sin).
+ * sentinel_oracle_rope_rotate: rotates the (even, odd) row pairs of every head in place
+ * (Layers/RotaryEmbedding.cpp:39-59; inverse :61-81).  Column c of the `columns` columns
+ * starting at colStart uses table position  segmentLength > 0 ? c % segmentLength :
+ * positionOffset + c  (the device rule, Cuda/CudaOps.cu:362-402; the host layer is the
+ * case positionOffset = 0, segmentLength = 0).  Returns -1 on invalid geometry or a
+ * position past the table (Cuda/CudaOps.cu:1319-1330).
+ * Pinned bit-exactly against the reference's compiled RotaryEmbedding (tests/golden,
+ * tests/test_oracle_rope.py) and by rotation invariants.
+ */
+int sentinel_oracle_rope_tables(int headDim, int positions, float base, float* cosTable, float* sinTable);
+int sentinel_oracle_rope_rotate(float* tensor, int heads, int headDim, int strideColumns, int colStart, int columns,
+                                int positionOffset, int segmentLength, const float* cosTable, const float* sinTable,
+                                int tablePositions, int inverse);
+
 int sentinel_oracle_max_threads(void);
 
 #ifdef __cplusplus

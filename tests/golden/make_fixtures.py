@@ -69,6 +69,21 @@ def main():
     np.savez_compressed(os.path.join(HERE, "gemm_softmax_kat.npz"), **kat)
     print("gemm_softmax_kat", len(kat), "arrays")
 
+    # RoPE tables and rotations from the reference's RotaryEmbedding (Layers/RotaryEmbedding.cpp)
+    rng = np.random.default_rng(0x5E17 + 30)
+    rope = {}
+    for tag, (heads, d, t, base) in {"h3_d16_T40": (3, 16, 40, 10000.0), "h2_d64_T130": (2, 64, 130, 10000.0),
+                                     "h1_d128_T33_base500k": (1, 128, 33, 500000.0)}.items():
+        x = rng.standard_normal((heads * d, t)).astype(np.float32)
+        cos, sin = oracle_lib.rope_tables(d, t + 7, base, lib="ref")
+        rope[f"{tag}_geometry"] = np.array([heads, d, t, t + 7], dtype=np.int64)
+        rope[f"{tag}_base"] = np.float32(base)
+        rope[f"{tag}_x"], rope[f"{tag}_cos"], rope[f"{tag}_sin"] = x, cos, sin
+        rope[f"{tag}_forward"] = oracle_lib.ref_rope_rotate(x, heads, d, t + 7, base)
+        rope[f"{tag}_inverse"] = oracle_lib.ref_rope_rotate(x, heads, d, t + 7, base, inverse=True)
+    np.savez_compressed(os.path.join(HERE, "rope_kat.npz"), **rope)
+    print("rope_kat", sorted(rope))
+
 
 if __name__ == "__main__":
     main()

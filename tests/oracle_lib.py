@@ -46,6 +46,8 @@ def oracle():
         lib.sentinel_oracle_gemm.argtypes = [_fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int]
         lib.sentinel_oracle_softmax_columns.argtypes = [_fp, _fp, ctypes.c_int, ctypes.c_int]
         lib.sentinel_oracle_max_threads.restype = ctypes.c_int
+        lib.sentinel_oracle_rope_tables.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, _fp, _fp]
+        lib.sentinel_oracle_rope_rotate.argtypes = [_fp] + [ctypes.c_int] * 7 + [_fp, _fp, ctypes.c_int, ctypes.c_int]
         _oracle = lib
     return _oracle
 
@@ -60,6 +62,8 @@ def reference():
         lib.sentinel_ref_attention.argtypes = [_fp] * 9 + [ctypes.c_int] * 8
         lib.sentinel_ref_gemm.argtypes = [_fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int]
         lib.sentinel_ref_softmax_columns.argtypes = [_fp, _fp, ctypes.c_int, ctypes.c_int]
+        lib.sentinel_ref_rope_tables.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, _fp, _fp]
+        lib.sentinel_ref_rope_rotate.argtypes = [_fp] + [ctypes.c_int] * 4 + [ctypes.c_float, ctypes.c_int]
         _ref = lib
     return _ref
 
@@ -126,4 +130,35 @@ def softmax_columns(x, lib="oracle"):
     rc = fn(_ptr(x), _ptr(y), x.shape[0], x.shape[1])
     if rc != 0:
         raise ValueError(f"{lib} softmax returned {rc}")
+    return y
+
+
+def rope_tables(head_dim, positions, base=10000.0, lib="oracle"):
+    """cos / sin tables [positions, head_dim // 2] as RotaryEmbedding builds them."""
+    cos = np.empty((positions, head_dim // 2), dtype=np.float32)
+    sin = np.empty_like(cos)
+    fn = oracle().sentinel_oracle_rope_tables if lib == "oracle" else reference().sentinel_ref_rope_tables
+    if fn(head_dim, positions, float(base), _ptr(cos), _ptr(sin)) != 0:
+        raise ValueError("rope tables: invalid arguments")
+    return cos, sin
+
+
+def rope_rotate(x, heads, head_dim, cos, sin, *, col_start=0, columns=None, position_offset=0, segment_length=0,
+                inverse=False):
+    """Oracle RoPE on a copy of x ([(head*d + dim), stride] fp32); returns the rotated copy."""
+    y = np.ascontiguousarray(x, dtype=np.float32).copy()
+    columns = y.shape[1] - col_start if columns is None else columns
+    rc = oracle().sentinel_oracle_rope_rotate(_ptr(y), heads, head_dim, y.shape[1], col_start, columns, position_offset,
+                                              segment_length, _ptr(cos), _ptr(sin), cos.shape[0], int(inverse))
+    if rc != 0:
+        raise ValueError("rope rotate: invalid arguments")
+    return y
+
+
+def ref_rope_rotate(x, heads, head_dim, positions, base=10000.0, inverse=False):
+    """The compiled reference's RotaryEmbedding::rotate(Inverse)InPlace on a copy of x (column = position)."""
+    y = np.ascontiguousarray(x, dtype=np.float32).copy()
+    rc = reference().sentinel_ref_rope_rotate(_ptr(y), heads, head_dim, y.shape[1], positions, float(base), int(inverse))
+    if rc != 0:
+        raise ValueError("reference rope rotate: invalid arguments")
     return y
