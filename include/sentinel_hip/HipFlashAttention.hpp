@@ -221,5 +221,49 @@ private:
     }
 };
 
+/// The rotary-embedding pair of Sentinel's CudaOps (sentinel/NeuralNet/Cuda/CudaOps.hpp:155-159): same names,
+/// argument order, defaults and exceptions (Cuda/CudaOps.cu:1318-1360). Tables are rows = positions,
+/// cols = pairCount, as CudaCausalSelfAttention keeps them.
+class HipOps {
+public:
+    static void rotaryRotateInPlace(HipMatrix& tensor, int headCount, int headDimension, int pairCount,
+                                    const HipMatrix& cosTable, const HipMatrix& sinTable, int positionOffset = 0,
+                                    int segmentLength = 0) {
+        rotate("HipOps::rotaryRotateInPlace", tensor, headCount, headDimension, pairCount, cosTable, sinTable,
+               positionOffset, segmentLength, 0);
+    }
+    static void rotaryRotateInverseInPlace(HipMatrix& tensor, int headCount, int headDimension, int pairCount,
+                                           const HipMatrix& cosTable, const HipMatrix& sinTable, int positionOffset = 0,
+                                           int segmentLength = 0) {
+        rotate("HipOps::rotaryRotateInverseInPlace", tensor, headCount, headDimension, pairCount, cosTable, sinTable,
+               positionOffset, segmentLength, 1);
+    }
+
+private:
+    static void rotate(const char* op, HipMatrix& tensor, int headCount, int headDimension, int pairCount,
+                       const HipMatrix& cosTable, const HipMatrix& sinTable, int positionOffset, int segmentLength,
+                       int inverse) {
+        const std::string name(op);
+        if (tensor.empty()) throw std::invalid_argument(name + " empty tensor");
+        if (headCount <= 0 || headDimension <= 0 || pairCount <= 0 || 2 * pairCount != headDimension)
+            throw std::invalid_argument(name + " invalid rope dims");
+        if (static_cast<int>(tensor.rows) != headCount * headDimension) throw std::invalid_argument(name + " embedding dim mismatch");
+        if (cosTable.empty() || sinTable.empty()) throw std::invalid_argument(name + " empty tables");
+        if (cosTable.cols != static_cast<size_t>(pairCount) || sinTable.cols != cosTable.cols || sinTable.rows != cosTable.rows)
+            throw std::invalid_argument(name + " table shape mismatch");
+        if (!sentinel_hip_device_available()) throw std::runtime_error(name + " no HIP device");
+        const int code = sentinel_hip_rope_rotate(tensor.buffer.deviceData, headCount, headDimension,
+                                                  static_cast<int>(tensor.cols), 0, static_cast<int>(tensor.cols),
+                                                  positionOffset, segmentLength, cosTable.buffer.deviceData,
+                                                  sinTable.buffer.deviceData, static_cast<int>(cosTable.rows), inverse,
+                                                  HipFlashAttention::activeStream());
+        if (code == SENTINEL_HIP_OK) return;
+        std::string detail = sentinel_hip_last_error();
+        if (detail.empty()) detail = sentinel_hip_strerror(code);
+        if (code == SENTINEL_HIP_RUNTIME) throw std::runtime_error(detail);
+        throw std::invalid_argument(detail);
+    }
+};
+
 }  // namespace sentinel_hip_host
 #endif

@@ -100,6 +100,45 @@ SENTINEL_HIP_API int sentinel_hip_flash_bwd(const void* q, const void* k, const 
                            int column_start, int seq_len, int pack_count, float scale, int causal, void* workspace,
                            size_t workspace_bytes, void* stream);
 
+/*
+ * Rotary position embedding: the step on either side of the attention core.
+ *
+ * Tables are fp32 [table_positions][head_dim / 2] in device memory, row = position, as the caller keeps them
+ * in CudaCausalSelfAttention::cosTable / sinTable (built by RotaryEmbedding, Layers/RotaryEmbedding.cpp:8-29).
+ *
+ * sentinel_hip_rope_rotate rotates the (even, odd) row pairs of every head of an fp32 column-layout matrix in
+ * place. Column c of the `columns` columns from column_start uses table position
+ *      segment_length > 0 ? c % segment_length : position_offset + c.
+ * Replaces CudaOps::rotaryRotateInPlace (inverse = 0) and CudaOps::rotaryRotateInverseInPlace (inverse != 0)
+ * (Cuda/CudaOps.cu:362-402, host side :1318-1360), with their argument checks. The arithmetic is plain fp32
+ * multiply / add (no fused multiply-add), so results are bit-identical to the host RotaryEmbedding.
+ */
+SENTINEL_HIP_API int sentinel_hip_rope_rotate(float* tensor, int heads, int head_dim, int stride_columns, int column_start,
+                             int columns, int position_offset, int segment_length, const float* cos_table,
+                             const float* sin_table, int table_positions, int inverse, void* stream);
+
+/*
+ * sentinel_hip_flash_fwd / _bwd on UNROTATED q and k: token t of every pack is rotated with table row
+ * position_offset + t on the way into the kernels, and dq, dk come back rotated back (gradients with respect
+ * to the unrotated tensors). One call replaces the sequence the CUDA layer runs around the attention core:
+ * rotaryRotateInPlace(query), rotaryRotateInPlace(key) (Cuda/CudaCausalSelfAttention.cu:206-207), forwardMultiHead
+ * / backwardMultiHead, rotaryRotateInverseInPlace(queryGradient), (keyGradient) (:508-509), with
+ * segmentLength = seq_len. The rotation rides on the layout conversion, so these exist for the configuration
+ * that has one (COLUMNS layout, fp32 tensors, 16-bit arithmetic); anything else returns
+ * SENTINEL_HIP_UNSUPPORTED and the caller rotates with sentinel_hip_rope_rotate. Workspace as for the plain calls.
+ */
+SENTINEL_HIP_API int sentinel_hip_flash_fwd_rope(const void* q, const void* k, const void* v, void* out, float* lse,
+                                const float* cos_table, const float* sin_table, int table_positions, int position_offset,
+                                int io_dtype, int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+                                int stride_columns, int column_start, int seq_len, int pack_count, float scale, int causal,
+                                void* workspace, size_t workspace_bytes, void* stream);
+SENTINEL_HIP_API int sentinel_hip_flash_bwd_rope(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                                const void* d_out, void* dq, void* dk, void* dv, float* delta, const float* cos_table,
+                                const float* sin_table, int table_positions, int position_offset, int io_dtype,
+                                int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim, int stride_columns,
+                                int column_start, int seq_len, int pack_count, float scale, int causal, void* workspace,
+                                size_t workspace_bytes, void* stream);
+
 /* Largest head_dim any kernel here accepts (the CUDA path's CudaFlashAttention::maxHeadDimension is 64). */
 SENTINEL_HIP_API int sentinel_hip_flash_max_head_dim(void);
 

@@ -1,6 +1,7 @@
 """MI355X-native causal flash attention behind Sentinel's CudaFlashAttention interface."""
 from .flash_attention import (  # noqa: F401
     HipFlashAttention,
+    HipOps,
     collect_kernel_timings,
     flash_attention_backward,
     flash_attention_forward,

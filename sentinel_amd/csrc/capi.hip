@@ -174,16 +174,34 @@ extern "C" size_t sentinel_hip_flash_workspace_bytes(int io_dtype, int compute_d
     return workspace_need(r, backward != 0);
 }
 
-extern "C" int sentinel_hip_flash_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int io_dtype,
-                                      int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
-                                      int stride_columns, int column_start, int seq_len, int pack_count, float scale,
-                                      int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
-    const char* op = "sentinel_hip_flash_fwd";
+namespace {
+
+// Checks of the rotary tables shared by the fused entry points and sentinel_hip_rope_rotate; messages follow
+// CudaOps::rotaryRotateInPlace (Cuda/CudaOps.cu:1319-1330).
+int check_rope(const char* op, const float* cos_table, const float* sin_table, int table_positions, int head_dim,
+               int position_offset, int positions_needed) {
+    if (!cos_table || !sin_table || table_positions <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty tables", op);
+    if (head_dim <= 0 || head_dim % 2 != 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s invalid rope dims", op);
+    if (position_offset < 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s negative positionOffset", op);
+    if ((long long)position_offset + positions_needed > table_positions)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s position exceeds RoPE table", op);
+    return SENTINEL_HIP_OK;
+}
+
+int flash_fwd(const char* op, const void* q, const void* k, const void* v, void* out, float* lse, int io_dtype,
+              int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim, int stride_columns, int column_start,
+              int seq_len, int pack_count, float scale, int causal, void* workspace, size_t workspace_bytes,
+              void* stream_ptr, RopeTables rope) {
     if (!q || !k || !v || !out || !lse) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
     Resolved r;
     const int rc = resolve(op, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns, column_start,
                            seq_len, pack_count, scale, causal, &r);
     if (rc != SENTINEL_HIP_OK) return rc;
+    if (rope.cos && !r.adapter)
+        return fail(SENTINEL_HIP_UNSUPPORTED,
+                    "%s the rotation is fused into the layout conversion of fp32 column tensors with 16-bit arithmetic; "
+                    "rotate other tensors with sentinel_hip_rope_rotate",
+                    op);
     if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
     hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
     const AttnGeom& g = r.g;
@@ -217,34 +235,39 @@ extern "C" int sentinel_hip_flash_fwd(const void* q, const void* k, const void* 
     void* v16 = ws + 2 * q_bytes16(g) + kv_bytes16(g);
     const long long off = r.column_start;
     const int stride = static_cast<int>(r.stride);
+    const RopeTables none = {nullptr, nullptr, 0};
     hipError_t err = launch_columns_to_bhtd(type, static_cast<const float*>(q) + off, q16, g.q_heads, g.head_dim, stride,
-                                            g.seq_len, g.packs, stream);
+                                            g.seq_len, g.packs, rope, stream);
     if (err == hipSuccess)
         err = launch_columns_to_bhtd(type, static_cast<const float*>(k) + off, k16, g.kv_heads, g.head_dim, stride,
-                                     g.seq_len, g.packs, stream);
+                                     g.seq_len, g.packs, rope, stream);
     if (err == hipSuccess)
         err = launch_columns_to_bhtd(type, static_cast<const float*>(v) + off, v16, g.kv_heads, g.head_dim, stride,
-                                     g.seq_len, g.packs, stream);
+                                     g.seq_len, g.packs, none, stream);
     if (err == hipSuccess) err = launch_fwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g, stream);
     if (err == hipSuccess)
         err = launch_bhtd_to_columns(type, o16, static_cast<float*>(out) + off, g.q_heads, g.head_dim, stride, g.seq_len,
-                                     g.packs, stream);
+                                     g.packs, none, stream);
     if (err != hipSuccess) return fail_hip("MFMA forward (column layout) launch", err);
     return SENTINEL_HIP_OK;
 }
 
-extern "C" int sentinel_hip_flash_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
-                                      const void* d_out, void* dq, void* dk, void* dv, float* delta, int io_dtype,
-                                      int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
-                                      int stride_columns, int column_start, int seq_len, int pack_count, float scale,
-                                      int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
-    const char* op = "sentinel_hip_flash_bwd";
+
+int flash_bwd(const char* op, const void* q, const void* k, const void* v, const void* out, const float* lse,
+              const void* d_out, void* dq, void* dk, void* dv, float* delta, int io_dtype, int compute_dtype, int layout,
+              int q_heads, int kv_heads, int head_dim, int stride_columns, int column_start, int seq_len, int pack_count,
+              float scale, int causal, void* workspace, size_t workspace_bytes, void* stream_ptr, RopeTables rope) {
     if (!q || !k || !v || !out || !lse || !d_out || !dq || !dk || !dv || !delta)
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
     Resolved r;
     const int rc = resolve(op, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns, column_start,
                            seq_len, pack_count, scale, causal, &r);
     if (rc != SENTINEL_HIP_OK) return rc;
+    if (rope.cos && !r.adapter)
+        return fail(SENTINEL_HIP_UNSUPPORTED,
+                    "%s the rotation is fused into the layout conversion of fp32 column tensors with 16-bit arithmetic; "
+                    "rotate other tensors with sentinel_hip_rope_rotate",
+                    op);
     if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
     hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
     const AttnGeom& g = r.g;
@@ -287,31 +310,109 @@ extern "C" int sentinel_hip_flash_bwd(const void* q, const void* k, const void* 
     const long long off = r.column_start;
     const int stride = static_cast<int>(r.stride);
     const int T = g.seq_len;
+    const RopeTables none = {nullptr, nullptr, 0};
     hipError_t err = launch_columns_to_bhtd(type, static_cast<const float*>(q) + off, q16, g.q_heads, g.head_dim, stride, T,
-                                            g.packs, stream);
+                                            g.packs, rope, stream);
     if (err == hipSuccess)
         err = launch_columns_to_bhtd(type, static_cast<const float*>(out) + off, o16, g.q_heads, g.head_dim, stride, T,
-                                     g.packs, stream);
+                                     g.packs, none, stream);
     if (err == hipSuccess)
         err = launch_columns_to_bhtd(type, static_cast<const float*>(d_out) + off, g16, g.q_heads, g.head_dim, stride, T,
-                                     g.packs, stream);
+                                     g.packs, none, stream);
     if (err == hipSuccess)
         err = launch_columns_to_bhtd(type, static_cast<const float*>(k) + off, k16, g.kv_heads, g.head_dim, stride, T,
-                                     g.packs, stream);
+                                     g.packs, rope, stream);
     if (err == hipSuccess)
         err = launch_columns_to_bhtd(type, static_cast<const float*>(v) + off, v16, g.kv_heads, g.head_dim, stride, T,
-                                     g.packs, stream);
+                                     g.packs, none, stream);
     if (err == hipSuccess)
         err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream);
+    // gradients with respect to the unrotated Q, K: the inverse rotation rides on the way out
     if (err == hipSuccess)
         err = launch_bhtd_to_columns(type, dq16, static_cast<float*>(dq) + off, g.q_heads, g.head_dim, stride, T, g.packs,
-                                     stream);
+                                     rope, stream);
     if (err == hipSuccess)
         err = launch_bhtd_to_columns(type, dk16, static_cast<float*>(dk) + off, g.kv_heads, g.head_dim, stride, T, g.packs,
-                                     stream);
+                                     rope, stream);
     if (err == hipSuccess)
         err = launch_bhtd_to_columns(type, dv16, static_cast<float*>(dv) + off, g.kv_heads, g.head_dim, stride, T, g.packs,
-                                     stream);
+                                     none, stream);
     if (err != hipSuccess) return fail_hip("MFMA backward (column layout) launch", err);
+    return SENTINEL_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" int sentinel_hip_flash_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int io_dtype,
+                                      int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+                                      int stride_columns, int column_start, int seq_len, int pack_count, float scale,
+                                      int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
+    const RopeTables none = {nullptr, nullptr, 0};
+    return flash_fwd("sentinel_hip_flash_fwd", q, k, v, out, lse, io_dtype, compute_dtype, layout, q_heads, kv_heads,
+                     head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes,
+                     stream_ptr, none);
+}
+
+extern "C" int sentinel_hip_flash_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                                      const void* d_out, void* dq, void* dk, void* dv, float* delta, int io_dtype,
+                                      int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+                                      int stride_columns, int column_start, int seq_len, int pack_count, float scale,
+                                      int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
+    const RopeTables none = {nullptr, nullptr, 0};
+    return flash_bwd("sentinel_hip_flash_bwd", q, k, v, out, lse, d_out, dq, dk, dv, delta, io_dtype, compute_dtype, layout,
+                     q_heads, kv_heads, head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal,
+                     workspace, workspace_bytes, stream_ptr, none);
+}
+
+extern "C" int sentinel_hip_flash_fwd_rope(const void* q, const void* k, const void* v, void* out, float* lse,
+                                           const float* cos_table, const float* sin_table, int table_positions,
+                                           int position_offset, int io_dtype, int compute_dtype, int layout, int q_heads,
+                                           int kv_heads, int head_dim, int stride_columns, int column_start, int seq_len,
+                                           int pack_count, float scale, int causal, void* workspace,
+                                           size_t workspace_bytes, void* stream_ptr) {
+    const char* op = "sentinel_hip_flash_fwd_rope";
+    const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
+    if (rc != SENTINEL_HIP_OK) return rc;
+    const RopeTables rope = {cos_table, sin_table, position_offset};
+    return flash_fwd(op, q, k, v, out, lse, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns,
+                     column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes, stream_ptr, rope);
+}
+
+extern "C" int sentinel_hip_flash_bwd_rope(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                                           const void* d_out, void* dq, void* dk, void* dv, float* delta,
+                                           const float* cos_table, const float* sin_table, int table_positions,
+                                           int position_offset, int io_dtype, int compute_dtype, int layout, int q_heads,
+                                           int kv_heads, int head_dim, int stride_columns, int column_start, int seq_len,
+                                           int pack_count, float scale, int causal, void* workspace,
+                                           size_t workspace_bytes, void* stream_ptr) {
+    const char* op = "sentinel_hip_flash_bwd_rope";
+    const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
+    if (rc != SENTINEL_HIP_OK) return rc;
+    const RopeTables rope = {cos_table, sin_table, position_offset};
+    return flash_bwd(op, q, k, v, out, lse, d_out, dq, dk, dv, delta, io_dtype, compute_dtype, layout, q_heads, kv_heads,
+                     head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes,
+                     stream_ptr, rope);
+}
+
+extern "C" int sentinel_hip_rope_rotate(float* tensor, int heads, int head_dim, int stride_columns, int column_start,
+                                        int columns, int position_offset, int segment_length, const float* cos_table,
+                                        const float* sin_table, int table_positions, int inverse, void* stream_ptr) {
+    const char* op = inverse ? "sentinel_hip_rope_rotate (inverse)" : "sentinel_hip_rope_rotate";
+    if (!tensor) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty tensor", op);
+    if (heads <= 0 || head_dim <= 0 || head_dim % 2 != 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s invalid rope dims", op);
+    if (columns <= 0 || column_start < 0 || (long long)column_start + columns > stride_columns)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s column window outside the matrix", op);
+    if (segment_length < 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s segmentLength must be >= 0", op);
+    if (segment_length > 0 && segment_length > table_positions)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s segmentLength exceeds RoPE table", op);
+    const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, segment_length > 0 ? 0 : position_offset,
+                              segment_length > 0 ? segment_length : columns);
+    if (rc != SENTINEL_HIP_OK) return rc;
+    if (position_offset < 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s negative positionOffset", op);
+    if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
+    const hipError_t err = launch_rope_rotate_f32(tensor + column_start, heads, head_dim, stride_columns, columns,
+                                                  position_offset, segment_length, cos_table, sin_table, inverse != 0,
+                                                  static_cast<hipStream_t>(stream_ptr));
+    if (err != hipSuccess) return fail_hip("rope rotate launch", err);
     return SENTINEL_HIP_OK;
 }

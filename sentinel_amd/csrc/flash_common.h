@@ -56,10 +56,22 @@ hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* 
                            hipStream_t stream);
 
 // ---- layout adapter (layout_adapter.hip): Sentinel column layout fp32 <-> [B,H,T,d] bf16 / fp16 ----
+// Rotary embedding tables [positions][head_dim / 2] (cos == nullptr: no rotation); token t of a pack uses
+// table row offset + t.
+struct RopeTables {
+    const float* cos;
+    const float* sin;
+    int offset;
+};
+
 hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int heads, int head_dim, int stride_columns,
-                                  int seq_len, int packs, hipStream_t stream);
+                                  int seq_len, int packs, RopeTables rope, hipStream_t stream);
 hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,
-                                  int seq_len, int packs, hipStream_t stream);
+                                  int seq_len, int packs, RopeTables inverse_rope, hipStream_t stream);
+// in-place rotation of fp32 column-layout rows (tensor already advanced to the first column)
+hipError_t launch_rope_rotate_f32(float* tensor, int heads, int head_dim, int stride_columns, int columns,
+                                  int position_offset, int segment_length, const float* cos, const float* sin, bool inverse,
+                                  hipStream_t stream);
 
 // ---- optional per-kernel hipEvent timing (kernel_timing.hip) ----
 class KernelTimer {

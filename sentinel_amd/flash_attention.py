@@ -51,6 +51,12 @@ def load_library():
     lib.sentinel_hip_flash_fwd.restype = i
     lib.sentinel_hip_flash_bwd.argtypes = [vp] * 10 + [i] * 10 + [f, i, vp, sz, vp]
     lib.sentinel_hip_flash_bwd.restype = i
+    lib.sentinel_hip_flash_fwd_rope.argtypes = [vp] * 7 + [i] * 12 + [f, i, vp, sz, vp]
+    lib.sentinel_hip_flash_fwd_rope.restype = i
+    lib.sentinel_hip_flash_bwd_rope.argtypes = [vp] * 12 + [i] * 12 + [f, i, vp, sz, vp]
+    lib.sentinel_hip_flash_bwd_rope.restype = i
+    lib.sentinel_hip_rope_rotate.argtypes = [vp] + [i] * 7 + [vp, vp, i, i, vp]
+    lib.sentinel_hip_rope_rotate.restype = i
     lib.sentinel_hip_flash_workspace_bytes.argtypes = [i] * 9
     lib.sentinel_hip_flash_workspace_bytes.restype = sz
     lib.sentinel_hip_flash_max_head_dim.restype = i
@@ -118,6 +124,50 @@ def _workspace(lib, io, compute, layout, hq, hkv, d, t, packs, backward, device,
     return workspace, need
 
 
+def _rope_args(rope, head_dimension):
+    cos, sin = rope[0], rope[1]
+    offset = int(rope[2]) if len(rope) > 2 else 0
+    for t in (cos, sin):
+        if t is None or t.dim() != 2 or t.dtype != torch.float32 or not t.is_contiguous() or not t.is_cuda:
+            raise ValueError("rope tables must be contiguous fp32 device matrices [positions, head_dim / 2]")
+    if cos.shape != sin.shape or cos.shape[1] * 2 != head_dimension:
+        raise ValueError("rope tables must be [positions, head_dim / 2]")
+    return cos, sin, offset
+
+
+class HipOps:
+    """The two rotary-embedding entry points of Sentinel's CudaOps on MI355X (Cuda/CudaOps.hpp:155-159)."""
+
+    @staticmethod
+    def rotary_rotate_in_place(tensor, head_count, head_dimension, pair_count, cos_table, sin_table, position_offset=0,
+                               segment_length=0, *, inverse=False, stream=None):
+        """CudaOps::rotaryRotateInPlace: rotates the fp32 matrix [(head*d + dim), columns] in place."""
+        name = "HipOps::rotaryRotateInverseInPlace" if inverse else "HipOps::rotaryRotateInPlace"
+        if tensor is None or tensor.numel() == 0:
+            raise ValueError(f"{name} empty tensor")
+        if head_count <= 0 or head_dimension <= 0 or pair_count <= 0 or pair_count * 2 != head_dimension:
+            raise ValueError(f"{name} invalid rope dims")
+        if tensor.dim() != 2 or tensor.dtype != torch.float32 or not tensor.is_contiguous():
+            raise ValueError(f"{name} expects a contiguous fp32 matrix")
+        if tensor.shape[0] != head_count * head_dimension:
+            raise ValueError(f"{name} embedding dim mismatch")
+        if cos_table is None or sin_table is None or cos_table.numel() == 0 or sin_table.numel() == 0:
+            raise ValueError(f"{name} empty tables")
+        cos, sin, _ = _rope_args((cos_table, sin_table), head_dimension)
+        cols = int(tensor.shape[1])
+        _check(load_library().sentinel_hip_rope_rotate(_ptr(tensor), head_count, head_dimension, cols, 0, cols,
+                                                       int(position_offset), int(segment_length), _ptr(cos), _ptr(sin),
+                                                       int(cos.shape[0]), int(bool(inverse)), _stream_handle(stream)))
+        return tensor
+
+    @staticmethod
+    def rotary_rotate_inverse_in_place(tensor, head_count, head_dimension, pair_count, cos_table, sin_table,
+                                       position_offset=0, segment_length=0, *, stream=None):
+        """CudaOps::rotaryRotateInverseInPlace."""
+        return HipOps.rotary_rotate_in_place(tensor, head_count, head_dimension, pair_count, cos_table, sin_table,
+                                             position_offset, segment_length, inverse=True, stream=stream)
+
+
 class HipFlashAttention:
     """Static interface of Sentinel's CudaFlashAttention on MI355X."""
 
@@ -128,8 +178,11 @@ class HipFlashAttention:
     @staticmethod
     def forward_multi_head(query, key, value, out, log_sum_exp, head_count, head_dimension, scale, causal=True,
                            column_start=0, column_count=0, pack_count=1, *, kv_head_count=None, compute=None,
-                           workspace=None, stream=None):
-        """CudaFlashAttention::forwardMultiHead. Returns (out, log_sum_exp) (re-allocated if their shape was wrong)."""
+                           workspace=None, stream=None, rope=None):
+        """CudaFlashAttention::forwardMultiHead. Returns (out, log_sum_exp) (re-allocated if their shape was wrong).
+
+        rope = (cos_table, sin_table[, position_offset]): query and key are given unrotated and rotated on the way in
+        (the two rotaryRotateInPlace calls of CudaCausalSelfAttention.cu:206-207 fused into this call)."""
         lib = load_library()
         HipFlashAttention._validate(query, key, value, head_count, head_dimension, kv_head_count, "forwardMultiHead")
         kv_heads = head_count if kv_head_count in (None, 0) else kv_head_count
@@ -140,10 +193,14 @@ class HipFlashAttention:
         seq = column_count if column_count > 0 else cols - column_start
         ws, ws_bytes = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1),
                                   max(pack_count, 1), False, query.device, workspace)
-        _check(lib.sentinel_hip_flash_fwd(_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp), F32, comp,
-                                          LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start,
-                                          column_count, pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes,
-                                          _stream_handle(stream)))
+        tail = (F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start, column_count,
+                pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes, _stream_handle(stream))
+        if rope is None:
+            _check(lib.sentinel_hip_flash_fwd(_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp), *tail))
+        else:
+            cos, sin, offset = _rope_args(rope, head_dimension)
+            _check(lib.sentinel_hip_flash_fwd_rope(_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp),
+                                                   _ptr(cos), _ptr(sin), int(cos.shape[0]), offset, *tail))
         return out, log_sum_exp
 
     @staticmethod
@@ -156,8 +213,11 @@ class HipFlashAttention:
     def backward_multi_head(query, key, value, out, log_sum_exp, out_gradient, query_gradient, key_gradient,
                             value_gradient, delta_workspace, head_count, head_dimension, scale, causal=True,
                             column_start=0, column_count=0, pack_count=1, *, kv_head_count=None, compute=None,
-                            workspace=None, stream=None):
-        """CudaFlashAttention::backwardMultiHead. Returns (dQ, dK, dV, delta)."""
+                            workspace=None, stream=None, rope=None):
+        """CudaFlashAttention::backwardMultiHead. Returns (dQ, dK, dV, delta).
+
+        rope as in forward_multi_head: query / key unrotated, dQ / dK come back rotated back
+        (rotaryRotateInverseInPlace of CudaCausalSelfAttention.cu:508-509 fused into this call)."""
         lib = load_library()
         HipFlashAttention._validate(query, key, value, head_count, head_dimension, kv_head_count, "backwardMultiHead")
         kv_heads = head_count if kv_head_count in (None, 0) else kv_head_count
@@ -177,12 +237,15 @@ class HipFlashAttention:
         comp = _COMPUTE_CODE[compute]
         ws, ws_bytes = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1), packs,
                                   True, query.device, workspace)
-        _check(lib.sentinel_hip_flash_bwd(_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp),
-                                          _ptr(out_gradient), _ptr(query_gradient), _ptr(key_gradient),
-                                          _ptr(value_gradient), _ptr(delta_workspace), F32, comp, LAYOUT_COLUMNS,
-                                          head_count, kv_heads, head_dimension, cols, column_start, column_count,
-                                          pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes,
-                                          _stream_handle(stream)))
+        head = (_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp), _ptr(out_gradient), _ptr(query_gradient),
+                _ptr(key_gradient), _ptr(value_gradient), _ptr(delta_workspace))
+        tail = (F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start, column_count,
+                pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes, _stream_handle(stream))
+        if rope is None:
+            _check(lib.sentinel_hip_flash_bwd(*head, *tail))
+        else:
+            cos, sin, offset = _rope_args(rope, head_dimension)
+            _check(lib.sentinel_hip_flash_bwd_rope(*head, _ptr(cos), _ptr(sin), int(cos.shape[0]), offset, *tail))
         return query_gradient, key_gradient, value_gradient, delta_workspace
 
     @staticmethod

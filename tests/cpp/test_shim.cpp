@@ -98,6 +98,29 @@ int main() {
         big.ensureSize(256, 8);
         big.fill(0.0f);
         expectInvalid("maxHeadDimension", [&] { HipFlashAttention::forwardMultiHead(big, big, big, out, lse, 1, 256, 0.25f); });
+        // rotary embedding: bit-identical to the oracle, inverse undoes it, reference exception on a short table
+        {
+            const int heads = 3, d = 32, cols = 70, positions = 80;
+            unsigned st = 7u;
+            auto hx = lcg(static_cast<size_t>(heads) * d * cols, st);
+            std::vector<float> hc(static_cast<size_t>(positions) * d / 2), hs(hc.size());
+            if (sentinel_oracle_rope_tables(d, positions, 10000.0f, hc.data(), hs.data()) != 0) throw std::runtime_error("oracle tables");
+            std::vector<float> want = hx;
+            if (sentinel_oracle_rope_rotate(want.data(), heads, d, cols, 0, cols, 5, 0, hc.data(), hs.data(), positions, 0) != 0)
+                throw std::runtime_error("oracle rope");
+            HipMatrix x, ct, stb;
+            x.upload(hx, static_cast<size_t>(heads) * d, cols);
+            ct.upload(hc, positions, d / 2);
+            stb.upload(hs, positions, d / 2);
+            HipOps::rotaryRotateInPlace(x, heads, d, d / 2, ct, stb, 5);
+            if (x.download() != want) throw std::runtime_error("rope rotate differs from the oracle");
+            HipOps::rotaryRotateInverseInPlace(x, heads, d, d / 2, ct, stb, 5);
+            const float back = maxAbsDiff(x.download(), hx, cols, 0, cols);
+            std::printf("  %-34s  bit-exact, inverse round trip %.2e\n", "rope H3 d32 T70 offset 5", back);
+            if (back > 2e-6f) throw std::runtime_error("rope inverse round trip");
+            expectInvalid("rope table too short", [&] { HipOps::rotaryRotateInPlace(x, heads, d, d / 2, ct, stb, 11); });
+            expectInvalid("rope dims", [&] { HipOps::rotaryRotateInPlace(x, heads, d, 0, ct, stb); });
+        }
         // single-head wrappers
         HipMatrix one, o1, l1, d1, d2, d3;
         one.ensureSize(16, 40);
