@@ -172,6 +172,78 @@ def cpu_baseline(name, heads_sample):
     }
 
 
+def columns_path(torch, name, steps, rope):
+    """The same step through Sentinel's own tensor layout (fp32 [(head*d + dim), B*T]) with 16-bit arithmetic:
+    what the drop-in costs on top of the kernels (layout / type conversion passes, optionally with the rotary
+    embedding fused into them instead of four separate elementwise passes)."""
+    import sentinel_amd
+    from sentinel_amd import HipFlashAttention, HipOps
+    b, hq, hkv, t, d, dtype, sigma, _ = CONFIGS[name]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5E17 + 40)
+    cols = b * t
+    q = sigma * torch.randn(hq * d, cols, device="cuda", generator=gen)
+    k = sigma * torch.randn(hkv * d, cols, device="cuda", generator=gen)
+    v = torch.randn(hkv * d, cols, device="cuda", generator=gen)
+    g = torch.randn(hq * d, cols, device="cuda", generator=gen)
+    pos = torch.arange(t, device="cuda", dtype=torch.float32)[:, None]
+    inv = torch.pow(torch.tensor(10000.0, device="cuda"), -2.0 * torch.arange(d // 2, device="cuda") / d)[None, :]
+    cos, sin = torch.cos(pos * inv).contiguous(), torch.sin(pos * inv).contiguous()
+    scale = 1.0 / d ** 0.5
+    args = (hq, d, scale, True, 0, t, b)
+    state = {"out": None, "lse": None, "dq": None, "dk": None, "dv": None, "delta": None, "ws": None}
+    lib = sentinel_amd.load_library()
+    need = lib.sentinel_hip_flash_workspace_bytes(0, {"bf16": 1, "fp16": 2}[dtype], 0, hq, hkv, d, t, b, 1)
+    state["ws"] = torch.empty(need, dtype=torch.uint8, device="cuda")
+
+    def step(mode):
+        kw = dict(kv_head_count=hkv, compute=dtype, workspace=state["ws"])
+        if mode == "fused":
+            kw["rope"] = (cos, sin)
+        if mode == "separate":  # the reference's sequence: rotate Q, K in place, attend, rotate dQ, dK back
+            HipOps.rotary_rotate_in_place(q, hq, d, d // 2, cos, sin, 0, t)
+            HipOps.rotary_rotate_in_place(k, hkv, d, d // 2, cos, sin, 0, t)
+        state["out"], state["lse"] = HipFlashAttention.forward_multi_head(q, k, v, state["out"], state["lse"], *args, **kw)
+        state["dq"], state["dk"], state["dv"], state["delta"] = HipFlashAttention.backward_multi_head(
+            q, k, v, state["out"], state["lse"], g, state["dq"], state["dk"], state["dv"], state["delta"], *args, **kw)
+        if mode == "separate":
+            HipOps.rotary_rotate_inverse_in_place(state["dq"], hq, d, d // 2, cos, sin, 0, t)
+            HipOps.rotary_rotate_inverse_in_place(state["dk"], hkv, d, d // 2, cos, sin, 0, t)
+            HipOps.rotary_rotate_inverse_in_place(q, hq, d, d // 2, cos, sin, 0, t)  # restore the inputs
+            HipOps.rotary_rotate_inverse_in_place(k, hkv, d, d // 2, cos, sin, 0, t)
+
+    report = {}
+    modes = ("plain", "fused", "separate") if rope else ("plain",)
+    for mode in modes:
+        for _ in range(2):
+            step(mode)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(mode)
+        torch.cuda.synchronize()
+        report[mode + "_ms_per_step"] = (time.perf_counter() - t0) / steps * 1e3
+    sentinel_amd.set_kernel_timing(True)
+    sentinel_amd.collect_kernel_timings()
+    for _ in range(steps):
+        step("fused" if rope else "plain")
+    times = sentinel_amd.collect_kernel_timings()
+    sentinel_amd.set_kernel_timing(False)
+    report["kernels_ms"] = {kname: tot / max(n, 1) for kname, (tot, n) in times.items()}
+    # conversion passes move 4 + 2 bytes per element; the in-place rotation 4 + 4
+    elems = float(hq * d) * cols
+    for kname, per_elem in (("columns_to_bhtd", 6.0), ("bhtd_to_columns", 6.0)):
+        if kname in times:
+            tot, n = times[kname]
+            # launches mix Q-sized and K/V-sized tensors: count the bytes of all of them
+            q_like = 3 + 1  # q, out, d_out in; dq out (+ q in, out out in the forward)
+            report[kname + "_avg_ms"] = tot / max(n, 1)
+    report["note"] = ("separate = rotate Q, K in place + plain step + rotate dQ, dK back (+ restoring Q, K: 4 extra passes "
+                      "that a real caller does not need); fused = rotation inside the conversion passes")
+    report["elements_per_q_tensor"] = elems
+    return report
+
+
 def rocminfo_gpu_clock_ghz():
     """Max Clock Freq. of the first gfx agent as printed by rocminfo (GHz), 0.0 if it cannot be read."""
     import re
@@ -196,6 +268,9 @@ def main():
     ap.add_argument("--config", default="nstar", choices=sorted(CONFIGS))
     ap.add_argument("--cpu-heads", type=int, default=8, help="(batch, head) pairs in the CPU baseline sample; 0 = skip")
     ap.add_argument("--no-configs", action="store_true", help="skip the brief timing of the other configurations")
+    ap.add_argument("--columns-path", action="store_true",
+                    help="also time the step through Sentinel's fp32 column layout (conversion passes, fused rotary "
+                         "embedding) and report it under \"columns_path\"")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB -> 1 GiB elementwise copy kernel three times, so that a counter run "
                          "(FETCH_SIZE / WRITE_SIZE) of this command holds a kernel of known traffic to scale by")
@@ -293,6 +368,11 @@ def main():
             del o
             torch.cuda.empty_cache()
         line["configs"] = others
+
+    if args.columns_path:
+        del w
+        torch.cuda.empty_cache()
+        line["columns_path"] = columns_path(torch, args.config, max(args.steps // 5, 3), rope=True)
 
     if args.cpu_heads > 0:
         line["cpu_baseline"] = cpu_baseline(args.config, args.cpu_heads)

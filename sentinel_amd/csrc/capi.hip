@@ -373,6 +373,8 @@ extern "C" int sentinel_hip_flash_fwd_rope(const void* q, const void* k, const v
     const char* op = "sentinel_hip_flash_fwd_rope";
     const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
     if (rc != SENTINEL_HIP_OK) return rc;
+    if (misaligned(cos_table) || misaligned(sin_table))
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
     const RopeTables rope = {cos_table, sin_table, position_offset};
     return flash_fwd(op, q, k, v, out, lse, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns,
                      column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes, stream_ptr, rope);
@@ -388,6 +390,8 @@ extern "C" int sentinel_hip_flash_bwd_rope(const void* q, const void* k, const v
     const char* op = "sentinel_hip_flash_bwd_rope";
     const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
     if (rc != SENTINEL_HIP_OK) return rc;
+    if (misaligned(cos_table) || misaligned(sin_table))
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
     const RopeTables rope = {cos_table, sin_table, position_offset};
     return flash_bwd(op, q, k, v, out, lse, d_out, dq, dk, dv, delta, io_dtype, compute_dtype, layout, q_heads, kv_heads,
                      head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes,

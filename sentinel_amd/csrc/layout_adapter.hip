@@ -36,7 +36,11 @@ __device__ __forceinline__ void rotate_pair(float& even, float& odd, float c, fl
     }
 }
 
-template <typename E>
+// Tile = 64 head dims x 64 tokens, kept in LDS as tile[dim][token] with a row stride of 65 floats: the
+// token-major side (fp32, 4 tokens per thread) and the dim-major side (16 bit, 8 dims = 16 bytes per thread)
+// both touch 64 different banks per wavefront access.  VEC4: the fp32 rows can be accessed as aligned float4
+// (pointer, stride and sequence length all multiples of 4 floats); otherwise the same code runs on scalars.
+template <typename E, bool VEC4>
 __global__ __launch_bounds__(256) void columns_to_bhtd_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst,
                                                                int heads, int d, long long stride, int T, RopeTables rope) {
     __shared__ float tile[kTile][kTile + 1];
@@ -45,30 +49,56 @@ __global__ __launch_bounds__(256) void columns_to_bhtd_kernel(const float* __res
     const int b = blockIdx.z / heads;
     const int h = blockIdx.z % heads;
     const int tid = threadIdx.x;
-    for (int i = 0; i < kTile * kTile / 256; ++i) {
-        const int c = i * 4 + tid / kTile;
-        const int t = tid % kTile;
-        float x = 0.0f;
-        if (t0 + t < T && c0 + c < d) x = src[((long long)h * d + c0 + c) * stride + (long long)b * T + t0 + t];
-        tile[c][t] = x;
+    {
+        const int t4 = (tid % 16) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = i * 16 + tid / 16;
+            float x[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (c0 + c < d) {
+                const float* at = src + ((long long)h * d + c0 + c) * stride + (long long)b * T + t0 + t4;
+                if (VEC4) {
+                    if (t0 + t4 < T) {
+                        const float4 v = *reinterpret_cast<const float4*>(at);
+                        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (t0 + t4 + e < T) x[e] = at[e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) tile[c][t4 + e] = x[e];
+        }
     }
     __syncthreads();
-    for (int i = 0; i < kTile * kTile / 512; ++i) {
-        const int t = i * 8 + tid / 32;
-        const int c = (tid % 32) * 2;
-        if (t0 + t < T && c0 + c < d) {
-            float even = tile[c][t];
-            float odd = tile[c + 1][t];
+    const int c8 = (tid % 8) * 8;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int t = i * 32 + tid / 8;
+        if (t0 + t < T && c0 + c8 < d) {
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = tile[c8 + e][t];
             if (rope.cos) {
-                const long long at = (long long)(rope.offset + t0 + t) * (d / 2) + (c0 + c) / 2;
-                rotate_pair<false>(even, odd, rope.cos[at], rope.sin[at]);
+                const long long at = (long long)(rope.offset + t0 + t) * (d / 2) + (c0 + c8) / 2;
+                const float4 c = *reinterpret_cast<const float4*>(rope.cos + at);
+                const float4 sn = *reinterpret_cast<const float4*>(rope.sin + at);
+                rotate_pair<false>(x[0], x[1], c.x, sn.x);
+                rotate_pair<false>(x[2], x[3], c.y, sn.y);
+                rotate_pair<false>(x[4], x[5], c.z, sn.z);
+                rotate_pair<false>(x[6], x[7], c.w, sn.w);
             }
-            *reinterpret_cast<unsigned*>(dst + (((long long)b * heads + h) * T + t0 + t) * d + c0 + c) = E::pack2(even, odd);
+            u32x4 w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = E::pack2(x[2 * e], x[2 * e + 1]);
+            *reinterpret_cast<u32x4*>(dst + (((long long)b * heads + h) * T + t0 + t) * d + c0 + c8) = w;
         }
     }
 }
 
-template <typename E>
+template <typename E, bool VEC4>
 __global__ __launch_bounds__(256) void bhtd_to_columns_kernel(const unsigned short* __restrict__ src, float* __restrict__ dst,
                                                                int heads, int d, long long stride, int T, RopeTables rope) {
     __shared__ float tile[kTile][kTile + 1];
@@ -77,26 +107,45 @@ __global__ __launch_bounds__(256) void bhtd_to_columns_kernel(const unsigned sho
     const int b = blockIdx.z / heads;
     const int h = blockIdx.z % heads;
     const int tid = threadIdx.x;
-    for (int i = 0; i < kTile * kTile / 512; ++i) {
-        const int t = i * 8 + tid / 32;
-        const int c = (tid % 32) * 2;
-        if (t0 + t < T && c0 + c < d) {
-            const unsigned w = *reinterpret_cast<const unsigned*>(src + (((long long)b * heads + h) * T + t0 + t) * d + c0 + c);
-            float even = E::lo(w);
-            float odd = E::hi(w);
-            if (rope.cos) {
-                const long long at = (long long)(rope.offset + t0 + t) * (d / 2) + (c0 + c) / 2;
-                rotate_pair<true>(even, odd, rope.cos[at], rope.sin[at]);
+    const int c8 = (tid % 8) * 8;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int t = i * 32 + tid / 8;
+        if (t0 + t < T && c0 + c8 < d) {
+            const u32x4 w = *reinterpret_cast<const u32x4*>(src + (((long long)b * heads + h) * T + t0 + t) * d + c0 + c8);
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                x[2 * e] = E::lo(w[e]);
+                x[2 * e + 1] = E::hi(w[e]);
             }
-            tile[c][t] = even;
-            tile[c + 1][t] = odd;
+            if (rope.cos) {
+                const long long at = (long long)(rope.offset + t0 + t) * (d / 2) + (c0 + c8) / 2;
+                const float4 c = *reinterpret_cast<const float4*>(rope.cos + at);
+                const float4 sn = *reinterpret_cast<const float4*>(rope.sin + at);
+                rotate_pair<true>(x[0], x[1], c.x, sn.x);
+                rotate_pair<true>(x[2], x[3], c.y, sn.y);
+                rotate_pair<true>(x[4], x[5], c.z, sn.z);
+                rotate_pair<true>(x[6], x[7], c.w, sn.w);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) tile[c8 + e][t] = x[e];
         }
     }
     __syncthreads();
-    for (int i = 0; i < kTile * kTile / 256; ++i) {
-        const int c = i * 4 + tid / kTile;
-        const int t = tid % kTile;
-        if (t0 + t < T && c0 + c < d) dst[((long long)h * d + c0 + c) * stride + (long long)b * T + t0 + t] = tile[c][t];
+    const int t4 = (tid % 16) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = i * 16 + tid / 16;
+        if (c0 + c >= d) continue;
+        float* at = dst + ((long long)h * d + c0 + c) * stride + (long long)b * T + t0 + t4;
+        if (VEC4) {
+            if (t0 + t4 < T) *reinterpret_cast<float4*>(at) = make_float4(tile[c][t4], tile[c][t4 + 1], tile[c][t4 + 2], tile[c][t4 + 3]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (t0 + t4 + e < T) at[e] = tile[c][t4 + e];
+        }
     }
 }
 
@@ -138,19 +187,29 @@ hipError_t launch_rope_rotate_f32(float* tensor, int heads, int head_dim, int st
     return hipGetLastError();
 }
 
+// fp32 rows can be read / written as aligned float4
+static bool rows_vec4(const void* base, int stride_columns, int seq_len) {
+    return (reinterpret_cast<uintptr_t>(base) & 15u) == 0 && stride_columns % 4 == 0 && seq_len % 4 == 0;
+}
+
 hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int heads, int head_dim, int stride_columns,
                                   int seq_len, int packs, RopeTables rope, hipStream_t stream) {
     const dim3 grid((seq_len + kTile - 1) / kTile, (head_dim + kTile - 1) / kTile, packs * heads);
     auto out = static_cast<unsigned short*>(dst);
+    if (head_dim % 8 != 0) return hipErrorInvalidValue;
+    const bool v4 = rows_vec4(src, stride_columns, seq_len);
     KernelTimer timer("columns_to_bhtd", stream);
-    if (type == Elem::BF16)
-        hipLaunchKernelGGL(columns_to_bhtd_kernel<Bf16>, grid, dim3(256), 0, stream, src, out, heads, head_dim,
-                           (long long)stride_columns, seq_len, rope);
-    else if (type == Elem::F16)
-        hipLaunchKernelGGL(columns_to_bhtd_kernel<Fp16>, grid, dim3(256), 0, stream, src, out, heads, head_dim,
-                           (long long)stride_columns, seq_len, rope);
-    else
+#define SENTINEL_LAUNCH(E, V) \
+    hipLaunchKernelGGL((columns_to_bhtd_kernel<E, V>), grid, dim3(256), 0, stream, src, out, heads, head_dim, \
+                       (long long)stride_columns, seq_len, rope)
+    if (type == Elem::BF16) {
+        if (v4) SENTINEL_LAUNCH(Bf16, true); else SENTINEL_LAUNCH(Bf16, false);
+    } else if (type == Elem::F16) {
+        if (v4) SENTINEL_LAUNCH(Fp16, true); else SENTINEL_LAUNCH(Fp16, false);
+    } else {
         return hipErrorInvalidValue;
+    }
+#undef SENTINEL_LAUNCH
     return hipGetLastError();
 }
 
@@ -158,15 +217,20 @@ hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int he
                                   int seq_len, int packs, RopeTables rope, hipStream_t stream) {
     const dim3 grid((seq_len + kTile - 1) / kTile, (head_dim + kTile - 1) / kTile, packs * heads);
     auto in = static_cast<const unsigned short*>(src);
+    if (head_dim % 8 != 0) return hipErrorInvalidValue;
+    const bool v4 = rows_vec4(dst, stride_columns, seq_len);
     KernelTimer timer("bhtd_to_columns", stream);
-    if (type == Elem::BF16)
-        hipLaunchKernelGGL(bhtd_to_columns_kernel<Bf16>, grid, dim3(256), 0, stream, in, dst, heads, head_dim,
-                           (long long)stride_columns, seq_len, rope);
-    else if (type == Elem::F16)
-        hipLaunchKernelGGL(bhtd_to_columns_kernel<Fp16>, grid, dim3(256), 0, stream, in, dst, heads, head_dim,
-                           (long long)stride_columns, seq_len, rope);
-    else
+#define SENTINEL_LAUNCH(E, V) \
+    hipLaunchKernelGGL((bhtd_to_columns_kernel<E, V>), grid, dim3(256), 0, stream, in, dst, heads, head_dim, \
+                       (long long)stride_columns, seq_len, rope)
+    if (type == Elem::BF16) {
+        if (v4) SENTINEL_LAUNCH(Bf16, true); else SENTINEL_LAUNCH(Bf16, false);
+    } else if (type == Elem::F16) {
+        if (v4) SENTINEL_LAUNCH(Fp16, true); else SENTINEL_LAUNCH(Fp16, false);
+    } else {
         return hipErrorInvalidValue;
+    }
+#undef SENTINEL_LAUNCH
     return hipGetLastError();
 }
 
