@@ -198,3 +198,35 @@ extern "C" int sentinel_ref_rope_rotate(float* tensor, int heads, int headDim, i
         return -1;
     }
 }
+
+// The reference's attention layer with real weights and its own RoPE tables, full causal mask (windowSize 0):
+// forward and, when d_y != NULL, backward. Shapes as in sentinel_oracle_layer.
+extern "C" int sentinel_ref_layer(const float* x, const float* wq, const float* wk, const float* wv, const float* wo,
+                                  const float* d_y, float* y, float* d_x, float* d_wq, float* d_wk, float* d_wv, float* d_wo,
+                                  int embeddingDim, int qHeads, int kvHeads, int headDim, int seqLen, float ropeBase,
+                                  int ropePositions) {
+    try {
+        const size_t e = static_cast<size_t>(embeddingDim), t = static_cast<size_t>(seqLen);
+        const size_t qRows = static_cast<size_t>(qHeads) * headDim, kvRows = static_cast<size_t>(kvHeads) * headDim;
+        auto load = [](const float* src, size_t rows, size_t cols) {
+            Matrix m(rows, cols, 0.0f);
+            std::copy(src, src + rows * cols, m.data.begin());
+            return m;
+        };
+        auto store = [](const Matrix& m, float* dst) { std::copy(m.data.begin(), m.data.end(), dst); };
+        CausalSelfAttention layer(load(wq, qRows, e), load(wk, kvRows, e), load(wv, kvRows, e), load(wo, e, qRows),
+                                  RotaryEmbedding(headDim, ropePositions, ropeBase), qHeads, 0, 0, kvHeads);
+        CausalSelfAttentionCache cache;
+        store(layer.forward(load(x, e, t), cache), y);
+        if (!d_y) return 0;
+        Matrix gwq, gwk, gwv, gwo;
+        store(layer.backward(load(d_y, e, t), cache, gwq, gwk, gwv, gwo), d_x);
+        store(gwq, d_wq);
+        store(gwk, d_wk);
+        store(gwv, d_wv);
+        store(gwo, d_wo);
+        return 0;
+    } catch (const std::exception&) {
+        return -1;
+    }
+}

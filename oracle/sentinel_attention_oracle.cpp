@@ -380,6 +380,58 @@ extern "C" int sentinel_oracle_rope_rotate(float* tensor, int heads, int headDim
     return 0;
 }
 
+// Layers/CausalSelfAttention.cpp:212-264 (forward) and :266-368 (backward), full causal mask
+extern "C" int sentinel_oracle_layer(const float* x, const float* wq, const float* wk, const float* wv, const float* wo,
+                                     const float* d_y, float* y, float* d_x, float* d_wq, float* d_wk, float* d_wv,
+                                     float* d_wo, int embeddingDim, int qHeads, int kvHeads, int headDim, int seqLen,
+                                     float ropeBase, int ropePositions) {
+    if (!x || !wq || !wk || !wv || !wo || !y) return -1;
+    if (embeddingDim <= 0 || qHeads <= 0 || kvHeads <= 0 || qHeads % kvHeads != 0 || headDim <= 0 || headDim % 2 != 0) return -1;
+    if (seqLen <= 0 || seqLen > ropePositions) return -1;
+    const bool wantBackward = d_y != nullptr;
+    if (wantBackward && (!d_x || !d_wq || !d_wk || !d_wv || !d_wo)) return -1;
+    const int e = embeddingDim, t = seqLen, qRows = qHeads * headDim, kvRows = kvHeads * headDim;
+    std::vector<float> cosT(static_cast<size_t>(ropePositions) * headDim / 2), sinT(cosT.size());
+    if (sentinel_oracle_rope_tables(headDim, ropePositions, ropeBase, cosT.data(), sinT.data()) != 0) return -1;
+
+    std::vector<float> q(static_cast<size_t>(qRows) * t), k(static_cast<size_t>(kvRows) * t), v(k.size()), a(q.size());
+    sentinel_oracle_gemm(wq, qRows, e, x, e, t, q.data(), 0, 0);
+    sentinel_oracle_gemm(wk, kvRows, e, x, e, t, k.data(), 0, 0);
+    sentinel_oracle_gemm(wv, kvRows, e, x, e, t, v.data(), 0, 0);
+    sentinel_oracle_rope_rotate(q.data(), qHeads, headDim, t, 0, t, 0, 0, cosT.data(), sinT.data(), ropePositions, 0);
+    sentinel_oracle_rope_rotate(k.data(), kvHeads, headDim, t, 0, t, 0, 0, cosT.data(), sinT.data(), ropePositions, 0);
+    const float scale = 1.0f / std::sqrt(static_cast<float>(headDim));
+    if (!wantBackward) {
+        if (sentinel_oracle_attention(q.data(), k.data(), v.data(), a.data(), nullptr, nullptr, nullptr, nullptr, nullptr,
+                                      qHeads, kvHeads, headDim, t, 0, t, 1, scale, 1, 0) != 0)
+            return -1;
+        sentinel_oracle_gemm(wo, e, qRows, a.data(), qRows, t, y, 0, 0);
+        return 0;
+    }
+    std::vector<float> dA(q.size()), dq(q.size()), dk(k.size()), dv(k.size()), temp(static_cast<size_t>(e) * t);
+    // forward once for A (and Y), then the backward from dA = Wo^T dY
+    if (sentinel_oracle_attention(q.data(), k.data(), v.data(), a.data(), nullptr, nullptr, nullptr, nullptr, nullptr, qHeads,
+                                  kvHeads, headDim, t, 0, t, 1, scale, 1, 0) != 0)
+        return -1;
+    sentinel_oracle_gemm(wo, e, qRows, a.data(), qRows, t, y, 0, 0);
+    sentinel_oracle_gemm(d_y, e, t, a.data(), qRows, t, d_wo, 0, 1);
+    sentinel_oracle_gemm(wo, e, qRows, d_y, e, t, dA.data(), 1, 0);
+    if (sentinel_oracle_attention(q.data(), k.data(), v.data(), a.data(), nullptr, dA.data(), dq.data(), dk.data(), dv.data(),
+                                  qHeads, kvHeads, headDim, t, 0, t, 1, scale, 1, 0) != 0)
+        return -1;
+    sentinel_oracle_rope_rotate(dq.data(), qHeads, headDim, t, 0, t, 0, 0, cosT.data(), sinT.data(), ropePositions, 1);
+    sentinel_oracle_rope_rotate(dk.data(), kvHeads, headDim, t, 0, t, 0, 0, cosT.data(), sinT.data(), ropePositions, 1);
+    sentinel_oracle_gemm(dq.data(), qRows, t, x, e, t, d_wq, 0, 1);
+    sentinel_oracle_gemm(dk.data(), kvRows, t, x, e, t, d_wk, 0, 1);
+    sentinel_oracle_gemm(dv.data(), kvRows, t, x, e, t, d_wv, 0, 1);
+    sentinel_oracle_gemm(wq, qRows, e, dq.data(), qRows, t, d_x, 1, 0);
+    sentinel_oracle_gemm(wk, kvRows, e, dk.data(), kvRows, t, temp.data(), 1, 0);
+    for (size_t i = 0; i < temp.size(); ++i) d_x[i] += temp[i];
+    sentinel_oracle_gemm(wv, kvRows, e, dv.data(), kvRows, t, temp.data(), 1, 0);
+    for (size_t i = 0; i < temp.size(); ++i) d_x[i] += temp[i];
+    return 0;
+}
+
 extern "C" int sentinel_oracle_max_threads(void) {
 #if defined(_OPENMP)
     return omp_get_max_threads();

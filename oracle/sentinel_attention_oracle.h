@@ -75,6 +75,24 @@ int sentinel_oracle_rope_rotate(float* tensor, int heads, int headDim, int strid
                                 int positionOffset, int segmentLength, const float* cosTable, const float* sinTable,
                                 int tablePositions, int inverse);
 
+/*
+ * The whole attention layer around the core, one sequence (embeddingDim x seqLen, row-major):
+ *   Q = Wq X, K = Wk X, V = Wv X; RoPE on Q and K; causal attention (scale 1/sqrt(headDim));
+ *   Y = Wo A                                              (Layers/CausalSelfAttention.cpp:212-264)
+ * and, when d_y != NULL, its backward                     (Layers/CausalSelfAttention.cpp:266-368):
+ *   dWo = dY A^T, dA = Wo^T dY, core backward, inverse RoPE on dQ, dK,
+ *   dWq = dQ X^T, dWk = dK X^T, dWv = dV X^T, dX = Wq^T dQ + Wk^T dK + Wv^T dV.
+ * wq: (qHeads*headDim) x E, wk / wv: (kvHeads*headDim) x E, wo: E x (qHeads*headDim); gradients have the
+ * shapes of what they differentiate. Composed from the functions above, so it inherits their pins; the
+ * composition itself is pinned bit-exactly against the reference's compiled layer (tests/golden/layer_kat.npz,
+ * tests/test_oracle_layer.py) and by finite differences.
+ * Returns 0, -1 on invalid geometry.
+ */
+int sentinel_oracle_layer(const float* x, const float* wq, const float* wk, const float* wv, const float* wo,
+                          const float* d_y, float* y, float* d_x, float* d_wq, float* d_wk, float* d_wv, float* d_wo,
+                          int embeddingDim, int qHeads, int kvHeads, int headDim, int seqLen, float ropeBase,
+                          int ropePositions);
+
 int sentinel_oracle_max_threads(void);
 
 #ifdef __cplusplus

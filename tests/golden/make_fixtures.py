@@ -84,6 +84,26 @@ def main():
     np.savez_compressed(os.path.join(HERE, "rope_kat.npz"), **rope)
     print("rope_kat", sorted(rope))
 
+    # the attention layer with real weights from the reference's CausalSelfAttention::forward / backward
+    rng = np.random.default_rng(0x5E17 + 40)
+    lay = {}
+    for tag, (e, hq, hkv, d, t, base) in {"e64_h4_T48": (64, 4, 4, 16, 48, 10000.0), "e48_gqa6q2kv_d8_T33": (48, 6, 2, 8, 33, 10000.0),
+                                          "e128_h2_d64_T70": (128, 2, 2, 64, 70, 500000.0)}.items():
+        bound = 1.0 / np.sqrt(e)
+        x = rng.standard_normal((e, t)).astype(np.float32)
+        wq = rng.uniform(-bound, bound, (hq * d, e)).astype(np.float32)
+        wk = rng.uniform(-bound, bound, (hkv * d, e)).astype(np.float32)
+        wv = rng.uniform(-bound, bound, (hkv * d, e)).astype(np.float32)
+        wo = rng.uniform(-bound, bound, (e, hq * d)).astype(np.float32)
+        d_y = rng.standard_normal((e, t)).astype(np.float32)
+        res = oracle_lib.layer(x, wq, wk, wv, wo, d_y, q_heads=hq, kv_heads=hkv, head_dim=d, rope_base=base,
+                               rope_positions=t + 3, lib="ref")
+        lay[f"{tag}_geometry"] = np.array([e, hq, hkv, d, t, t + 3], dtype=np.int64)
+        lay[f"{tag}_base"] = np.float32(base)
+        for key, val in dict(x=x, wq=wq, wk=wk, wv=wv, wo=wo, d_y=d_y, **res).items():
+            lay[f"{tag}_{key}"] = val
+    np.savez_compressed(os.path.join(HERE, "layer_kat.npz"), **lay)
+    print("layer_kat", len(lay), "arrays")
 
 if __name__ == "__main__":
     main()

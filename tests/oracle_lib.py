@@ -48,6 +48,7 @@ def oracle():
         lib.sentinel_oracle_max_threads.restype = ctypes.c_int
         lib.sentinel_oracle_rope_tables.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, _fp, _fp]
         lib.sentinel_oracle_rope_rotate.argtypes = [_fp] + [ctypes.c_int] * 7 + [_fp, _fp, ctypes.c_int, ctypes.c_int]
+        lib.sentinel_oracle_layer.argtypes = [_fp] * 12 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int]
         _oracle = lib
     return _oracle
 
@@ -64,6 +65,7 @@ def reference():
         lib.sentinel_ref_softmax_columns.argtypes = [_fp, _fp, ctypes.c_int, ctypes.c_int]
         lib.sentinel_ref_rope_tables.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, _fp, _fp]
         lib.sentinel_ref_rope_rotate.argtypes = [_fp] + [ctypes.c_int] * 4 + [ctypes.c_float, ctypes.c_int]
+        lib.sentinel_ref_layer.argtypes = [_fp] * 12 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int]
         _ref = lib
     return _ref
 
@@ -162,3 +164,25 @@ def ref_rope_rotate(x, heads, head_dim, positions, base=10000.0, inverse=False):
     if rc != 0:
         raise ValueError("reference rope rotate: invalid arguments")
     return y
+
+
+def layer(x, wq, wk, wv, wo, d_y=None, *, q_heads, kv_heads, head_dim, rope_base=10000.0, rope_positions=None,
+          lib="oracle"):
+    """The attention layer (projections, RoPE, causal attention, output projection) on one sequence x [E, T].
+
+    Returns dict(y[, d_x, d_wq, d_wk, d_wv, d_wo])."""
+    e, t = x.shape
+    rope_positions = t if rope_positions is None else rope_positions
+    y = np.empty((e, t), dtype=np.float32)
+    grads = [None] * 5
+    if d_y is not None:
+        grads = [np.empty_like(x), np.empty_like(wq), np.empty_like(wk), np.empty_like(wv), np.empty_like(wo)]
+    fn = oracle().sentinel_oracle_layer if lib == "oracle" else reference().sentinel_ref_layer
+    rc = fn(_ptr(x), _ptr(wq), _ptr(wk), _ptr(wv), _ptr(wo), _ptr(d_y), _ptr(y), *[_ptr(a) for a in grads], e, q_heads,
+            kv_heads, head_dim, t, float(rope_base), rope_positions)
+    if rc != 0:
+        raise ValueError(f"{lib} layer returned {rc}")
+    res = {"y": y}
+    if d_y is not None:
+        res.update(d_x=grads[0], d_wq=grads[1], d_wk=grads[2], d_wv=grads[3], d_wo=grads[4])
+    return res
