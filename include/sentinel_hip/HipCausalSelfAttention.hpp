@@ -1,0 +1,232 @@
+// Header-only C++ attention layer on the device for Sentinel's host code: the caller of the attention core.
+//
+// HipCausalSelfAttention mirrors the training-path face of class CudaCausalSelfAttention
+// (sentinel/NeuralNet/Cuda/CudaCausalSelfAttention.hpp:11-118): the same public weight / table / activation
+// members, uploadFrom, forward(input, out, segmentLength) and backward(outputGradient, inputGradient, four weight
+// gradients), so that a transformer block written against the CUDA class can hold this one instead. What it does
+// (Cuda/CudaCausalSelfAttention.cu:181-253 forward, :345-547 backward, flash branch):
+//   Q = Wq X, K = Wk X, V = Wv X        fp32 GEMMs (rocBLAS; the CUDA class uses cuBLASLt)
+//   RoPE on Q, K, packs restart at position 0 (segmentLength)
+//   flash attention, grouped-query heads read in place (no expandKvHeadsInto / reduceKvHeadGradsInto)
+//   Y = Wo A
+// and the backward of each step. With 16-bit HipFlashAttention::computeType() the rotation rides on the layout
+// conversion (sentinel_hip_flash_fwd_rope / _bwd_rope) and query / key stay unrotated in the cache; with fp32
+// arithmetic they are rotated in place like the reference's.
+// Not built: the dense materialising fallback (sliding-window / global-token masks, flash disabled), KV-cache
+// prefill / decode; those configurations throw std::runtime_error instead of running something else.
+// Link against libsentinel_hip_attn.so, rocBLAS and the HIP runtime.
+#ifndef SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
+#define SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
+
+#include "HipFlashAttention.hpp"
+
+#include <rocblas/rocblas.h>
+
+#include <cmath>
+
+namespace sentinel_hip_host {
+
+/// C = op(A) op(B) (+ C) on row-major fp32 device matrices; stands for CudaMatrix::multiplyInto and its
+/// transposed variants (sentinel/NeuralNet/Cuda/CudaMatmul.hpp).
+class HipGemm {
+public:
+    static void multiplyInto(const HipMatrix& a, const HipMatrix& b, HipMatrix& c, bool transposeA = false,
+                             bool transposeB = false, bool accumulate = false) {
+        const size_t m = transposeA ? a.cols : a.rows;
+        const size_t ka = transposeA ? a.rows : a.cols;
+        const size_t kb = transposeB ? b.cols : b.rows;
+        const size_t n = transposeB ? b.rows : b.cols;
+        if (a.empty() || b.empty() || ka != kb) throw std::invalid_argument("HipGemm::multiplyInto shape mismatch");
+        if (accumulate) {
+            if (c.rows != m || c.cols != n) throw std::invalid_argument("HipGemm::multiplyInto accumulate shape mismatch");
+        } else {
+            c.ensureSize(m, n);
+        }
+        const float alpha = 1.0f;
+        const float beta = accumulate ? 1.0f : 0.0f;
+        rocblas_handle h = handle();
+        if (rocblas_set_stream(h, HipFlashAttention::activeStream()) != rocblas_status_success)
+            throw std::runtime_error("HipGemm rocblas_set_stream failed");
+        // row-major C = op(A) op(B)  <=>  column-major C^T = op(B)^T op(A)^T, each row-major matrix read as its transpose
+        const rocblas_status st = rocblas_sgemm(
+            h, transposeB ? rocblas_operation_transpose : rocblas_operation_none,
+            transposeA ? rocblas_operation_transpose : rocblas_operation_none, static_cast<rocblas_int>(n),
+            static_cast<rocblas_int>(m), static_cast<rocblas_int>(ka), &alpha, b.buffer.deviceData,
+            static_cast<rocblas_int>(b.cols), a.buffer.deviceData, static_cast<rocblas_int>(a.cols), &beta,
+            c.buffer.deviceData, static_cast<rocblas_int>(n));
+        if (st != rocblas_status_success) throw std::runtime_error("HipGemm rocblas_sgemm failed");
+    }
+
+private:
+    static rocblas_handle handle() {
+        static rocblas_handle h = [] {
+            rocblas_handle created = nullptr;
+            if (rocblas_create_handle(&created) != rocblas_status_success) throw std::runtime_error("HipGemm rocblas_create_handle failed");
+            return created;
+        }();
+        return h;
+    }
+};
+
+/// What uploadFrom needs of the host layer (Layers/CausalSelfAttention.hpp:44-57): row-major weights
+/// (queryWeight (headCount*headDimension) x embeddingDim, key / value (kvHeadCount*headDimension) x embeddingDim,
+/// outputWeight embeddingDim x (headCount*headDimension)) and the RoPE parameters.
+struct HostAttentionWeights {
+    std::vector<float> queryWeight, keyWeight, valueWeight, outputWeight;
+    int embeddingDim = 0;
+    int headCount = 0;
+    int kvHeadCount = 0;  // <= 0: same as headCount
+    int headDimension = 0;
+    int maximumPositionCount = 0;
+    float ropeBase = 10000.0f;
+    int windowSize = 0;  // <= 0: full causal
+    int globalTokenCount = 0;
+};
+
+class HipCausalSelfAttention {
+public:
+    HipMatrix queryWeight, keyWeight, valueWeight, outputWeight;
+    HipMatrix cosTable, sinTable;
+    int headCount = 0;
+    int kvHeadCount = 0;
+    int headDimension = 0;
+    int pairCount = 0;
+    int maximumPositionCount = 0;
+    int windowSize = 0;
+    int globalTokenCount = 0;
+    int activeSegmentLength = 0;
+    int activePackCount = 0;
+    bool preferFlashAttention = true;
+    bool usedFlashAttention = false;
+
+    HipMatrix query, key, value, attended, output;
+    HipMatrix inputCache, attendedGradient, queryGradient, keyGradient, valueGradient;
+    HipMatrix flashLogSumExp, flashDelta;
+
+    /// upload weights and build the RoPE tables the way RotaryEmbedding does (Layers/RotaryEmbedding.cpp:8-29)
+    void uploadFrom(const HostAttentionWeights& host) {
+        const char* op = "HipCausalSelfAttention::uploadFrom";
+        if (host.embeddingDim <= 0 || host.headCount <= 0 || host.headDimension <= 0 || host.headDimension % 2 != 0)
+            throw std::invalid_argument(std::string(op) + " invalid dims");
+        const int kv = host.kvHeadCount <= 0 ? host.headCount : host.kvHeadCount;
+        if (host.headCount % kv != 0) throw std::invalid_argument(std::string(op) + " headCount must be divisible by kvHeadCount");
+        if (host.maximumPositionCount <= 0 || !(host.ropeBase > 0.0f)) throw std::invalid_argument(std::string(op) + " invalid rope");
+        headCount = host.headCount;
+        kvHeadCount = kv;
+        headDimension = host.headDimension;
+        pairCount = headDimension / 2;
+        maximumPositionCount = host.maximumPositionCount;
+        windowSize = host.windowSize;
+        globalTokenCount = host.globalTokenCount;
+        const size_t e = static_cast<size_t>(host.embeddingDim);
+        const size_t qRows = static_cast<size_t>(headCount) * headDimension, kvRows = static_cast<size_t>(kv) * headDimension;
+        queryWeight.upload(host.queryWeight, qRows, e);
+        keyWeight.upload(host.keyWeight, kvRows, e);
+        valueWeight.upload(host.valueWeight, kvRows, e);
+        outputWeight.upload(host.outputWeight, e, qRows);
+        std::vector<float> cosHost(static_cast<size_t>(maximumPositionCount) * pairCount), sinHost(cosHost.size());
+        for (int position = 0; position < maximumPositionCount; ++position)
+            for (int pairIndex = 0; pairIndex < pairCount; ++pairIndex) {
+                const float exponent = -2.0f * static_cast<float>(pairIndex) / static_cast<float>(headDimension);
+                const float angle = static_cast<float>(position) * std::pow(host.ropeBase, exponent);
+                cosHost[static_cast<size_t>(position) * pairCount + pairIndex] = std::cos(angle);
+                sinHost[static_cast<size_t>(position) * pairCount + pairIndex] = std::sin(angle);
+            }
+        cosTable.upload(cosHost, static_cast<size_t>(maximumPositionCount), static_cast<size_t>(pairCount));
+        sinTable.upload(sinHost, static_cast<size_t>(maximumPositionCount), static_cast<size_t>(pairCount));
+    }
+
+    static HipCausalSelfAttention createFrom(const HostAttentionWeights& host) {
+        HipCausalSelfAttention layer;
+        layer.uploadFrom(host);
+        return layer;
+    }
+
+    /// CudaCausalSelfAttention::canUseFlashAttention (Cuda/CudaCausalSelfAttention.cu:46-57) without the
+    /// multiple-of-4 rules, which these kernels do not need
+    bool canUseFlashAttention(int sequenceLength) const {
+        if (!preferFlashAttention) return false;
+        if (headDimension <= 0 || headDimension > HipFlashAttention::maxHeadDimension) return false;
+        if (windowSize > 0 && windowSize < sequenceLength) return false;
+        return true;
+    }
+
+    /// causal multi head attention writing into out; input is embeddingDim x columns, packs of segmentLength columns
+    void forward(const HipMatrix& input, HipMatrix& out, int segmentLength = 0) {
+        const char* op = "HipCausalSelfAttention::forward";
+        if (input.empty()) throw std::invalid_argument(std::string(op) + " empty input");
+        if (queryWeight.empty()) throw std::logic_error(std::string(op) + " called before uploadFrom");
+        if (queryWeight.cols != input.rows) throw std::invalid_argument(std::string(op) + " embedding dim mismatch");
+        const int columns = static_cast<int>(input.cols);
+        if (segmentLength <= 0) segmentLength = columns;
+        if (columns % segmentLength != 0) throw std::invalid_argument(std::string(op) + " columns must be a multiple of segmentLength");
+        if (segmentLength > maximumPositionCount) throw std::invalid_argument(std::string(op) + " segmentLength exceeds RoPE table");
+        if (!canUseFlashAttention(segmentLength))
+            throw std::runtime_error(std::string(op) + " needs the dense attention path (sparse window or flash disabled), which is not built");
+        activeSegmentLength = segmentLength;
+        activePackCount = columns / segmentLength;
+        usedFlashAttention = true;
+
+        inputCache.ensureSize(input.rows, input.cols);
+        throwIfHipFailed(hipMemcpyAsync(inputCache.buffer.deviceData, input.buffer.deviceData, input.byteCount(),
+                                        hipMemcpyDeviceToDevice, HipFlashAttention::activeStream()),
+                         "HipCausalSelfAttention::forward input copy");
+        HipGemm::multiplyInto(queryWeight, input, query);
+        HipGemm::multiplyInto(keyWeight, input, key);
+        HipGemm::multiplyInto(valueWeight, input, value);
+        const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
+        if (fusedRotation()) {
+            HipFlashAttention::forwardMultiHeadRope(query, key, value, attended, flashLogSumExp, cosTable, sinTable, 0, headCount,
+                                                    headDimension, scale, true, 0, segmentLength, activePackCount, kvHeadCount);
+        } else {
+            HipOps::rotaryRotateInPlace(query, headCount, headDimension, pairCount, cosTable, sinTable, 0, segmentLength);
+            HipOps::rotaryRotateInPlace(key, kvHeadCount, headDimension, pairCount, cosTable, sinTable, 0, segmentLength);
+            HipFlashAttention::forwardMultiHead(query, key, value, attended, flashLogSumExp, headCount, headDimension, scale, true,
+                                                0, segmentLength, activePackCount, kvHeadCount);
+        }
+        HipGemm::multiplyInto(outputWeight, attended, out);
+    }
+
+    /// backprop through the layer; weight gradients are overwritten (summed over all columns of the batch)
+    void backward(const HipMatrix& outputGradient, HipMatrix& inputGradient, HipMatrix& queryWeightGradient,
+                  HipMatrix& keyWeightGradient, HipMatrix& valueWeightGradient, HipMatrix& outputWeightGradient) {
+        const char* op = "HipCausalSelfAttention::backward";
+        if (inputCache.empty() || !usedFlashAttention) throw std::logic_error(std::string(op) + " called before forward");
+        if (outputGradient.rows != outputWeight.rows || outputGradient.cols != attended.cols)
+            throw std::invalid_argument(std::string(op) + " output gradient shape mismatch");
+        HipGemm::multiplyInto(outputGradient, attended, outputWeightGradient, false, true);
+        HipGemm::multiplyInto(outputWeight, outputGradient, attendedGradient, true, false);
+        const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
+        if (fusedRotation()) {
+            HipFlashAttention::backwardMultiHeadRope(query, key, value, attended, flashLogSumExp, attendedGradient, queryGradient,
+                                                     keyGradient, valueGradient, flashDelta, cosTable, sinTable, 0, headCount,
+                                                     headDimension, scale, true, 0, activeSegmentLength, activePackCount,
+                                                     kvHeadCount);
+        } else {
+            HipFlashAttention::backwardMultiHead(query, key, value, attended, flashLogSumExp, attendedGradient, queryGradient,
+                                                 keyGradient, valueGradient, flashDelta, headCount, headDimension, scale, true, 0,
+                                                 activeSegmentLength, activePackCount, kvHeadCount);
+            HipOps::rotaryRotateInverseInPlace(queryGradient, headCount, headDimension, pairCount, cosTable, sinTable, 0,
+                                               activeSegmentLength);
+            HipOps::rotaryRotateInverseInPlace(keyGradient, kvHeadCount, headDimension, pairCount, cosTable, sinTable, 0,
+                                               activeSegmentLength);
+        }
+        HipGemm::multiplyInto(queryGradient, inputCache, queryWeightGradient, false, true);
+        HipGemm::multiplyInto(keyGradient, inputCache, keyWeightGradient, false, true);
+        HipGemm::multiplyInto(valueGradient, inputCache, valueWeightGradient, false, true);
+        HipGemm::multiplyInto(queryWeight, queryGradient, inputGradient, true, false);
+        HipGemm::multiplyInto(keyWeight, keyGradient, inputGradient, true, false, true);
+        HipGemm::multiplyInto(valueWeight, valueGradient, inputGradient, true, false, true);
+    }
+
+private:
+    // the rotation rides on the fp32 <-> 16-bit conversion when there is one
+    bool fusedRotation() const {
+        const int compute = HipFlashAttention::computeType();
+        return (compute == SENTINEL_HIP_COMPUTE_BF16 || compute == SENTINEL_HIP_COMPUTE_F16) &&
+               (headDimension == 64 || headDimension == 128);
+    }
+};
+
+}  // namespace sentinel_hip_host
+#endif

@@ -1,0 +1,151 @@
+// GPU test of the C++ attention layer (include/sentinel_hip/HipCausalSelfAttention.hpp) against the CPU oracle's
+// layer, on the shapes of the reference's own device smoke tests (CudaCausalSelfAttention::runFlashParitySmokeDemo:
+// E=64, H=4, T=48; runGqaCudaSmokeDemo: grouped heads) plus packed batches and head_dim 64 / 128 with MFMA arithmetic.
+// Test infrastructure: the oracle is linked here only as the checker.
+#include "../../include/sentinel_hip/HipCausalSelfAttention.hpp"
+#include "../../oracle/sentinel_attention_oracle.h"
+
+#include <cmath>
+#include <cstdio>
+#include <stdexcept>
+#include <vector>
+
+using namespace sentinel_hip_host;
+
+static std::vector<float> lcg(size_t count, unsigned& state, float scale) {
+    std::vector<float> out(count);
+    for (size_t i = 0; i < count; ++i) {
+        state = state * 1664525u + 1013904223u;
+        out[i] = ((static_cast<float>(state >> 8) / 16777216.0f) * 2.0f - 1.0f) * scale;
+    }
+    return out;
+}
+
+static float relErr(const std::vector<float>& got, const std::vector<float>& want) {
+    float err = 0.0f, top = 0.0f;
+    for (size_t i = 0; i < got.size(); ++i) {
+        err = std::max(err, std::fabs(got[i] - want[i]));
+        top = std::max(top, std::fabs(want[i]));
+    }
+    return err / std::max(top, 1e-30f);
+}
+
+template <typename Fn>
+static void expectThrow(const char* what, Fn fn) {
+    try {
+        fn();
+    } catch (const std::exception&) {
+        return;
+    }
+    throw std::runtime_error(std::string("expected an exception: ") + what);
+}
+
+static void runCase(const char* name, int e, int heads, int kvHeads, int d, int T, int packs, int compute, float tol) {
+    const int qRows = heads * d, kvRows = kvHeads * d, cols = packs * T;
+    unsigned state = 2024u + static_cast<unsigned>(e + T);
+    const float bound = 1.0f / std::sqrt(static_cast<float>(e));
+    HostAttentionWeights host;
+    host.queryWeight = lcg(static_cast<size_t>(qRows) * e, state, bound);
+    host.keyWeight = lcg(static_cast<size_t>(kvRows) * e, state, bound);
+    host.valueWeight = lcg(static_cast<size_t>(kvRows) * e, state, bound);
+    host.outputWeight = lcg(static_cast<size_t>(e) * qRows, state, bound);
+    host.embeddingDim = e;
+    host.headCount = heads;
+    host.kvHeadCount = kvHeads;
+    host.headDimension = d;
+    host.maximumPositionCount = T + 5;
+    auto hx = lcg(static_cast<size_t>(e) * cols, state, 1.0f);
+    auto hg = lcg(static_cast<size_t>(e) * cols, state, 1.0f);
+
+    // oracle: one sequence at a time, weight gradients summed over the batch (what the train loop accumulates)
+    std::vector<float> wy(hx.size()), wdx(hx.size()), wdq(host.queryWeight.size(), 0.0f), wdk(host.keyWeight.size(), 0.0f),
+        wdv(host.valueWeight.size(), 0.0f), wdo(host.outputWeight.size(), 0.0f);
+    for (int p = 0; p < packs; ++p) {
+        std::vector<float> x(static_cast<size_t>(e) * T), g(x.size()), y(x.size()), dx(x.size()), dq(wdq.size()), dk(wdk.size()),
+            dv(wdv.size()), dwo(wdo.size());
+        for (int r = 0; r < e; ++r)
+            for (int c = 0; c < T; ++c) {
+                x[static_cast<size_t>(r) * T + c] = hx[static_cast<size_t>(r) * cols + p * T + c];
+                g[static_cast<size_t>(r) * T + c] = hg[static_cast<size_t>(r) * cols + p * T + c];
+            }
+        if (sentinel_oracle_layer(x.data(), host.queryWeight.data(), host.keyWeight.data(), host.valueWeight.data(),
+                                  host.outputWeight.data(), g.data(), y.data(), dx.data(), dq.data(), dk.data(), dv.data(),
+                                  dwo.data(), e, heads, kvHeads, d, T, host.ropeBase, host.maximumPositionCount) != 0)
+            throw std::runtime_error("oracle layer failed");
+        for (int r = 0; r < e; ++r)
+            for (int c = 0; c < T; ++c) {
+                wy[static_cast<size_t>(r) * cols + p * T + c] = y[static_cast<size_t>(r) * T + c];
+                wdx[static_cast<size_t>(r) * cols + p * T + c] = dx[static_cast<size_t>(r) * T + c];
+            }
+        for (size_t i = 0; i < wdq.size(); ++i) wdq[i] += dq[i];
+        for (size_t i = 0; i < wdk.size(); ++i) wdk[i] += dk[i];
+        for (size_t i = 0; i < wdv.size(); ++i) wdv[i] += dv[i];
+        for (size_t i = 0; i < wdo.size(); ++i) wdo[i] += dwo[i];
+    }
+
+    HipFlashAttention::computeType() = compute;
+    HipCausalSelfAttention layer = HipCausalSelfAttention::createFrom(host);
+    HipMatrix x, g, y, dx, dwq, dwk, dwv, dwo;
+    x.upload(hx, e, cols);
+    g.upload(hg, e, cols);
+    layer.forward(x, y, T);
+    layer.backward(g, dx, dwq, dwk, dwv, dwo);
+    const float ey = relErr(y.download(), wy), ex = relErr(dx.download(), wdx), eq = relErr(dwq.download(), wdq),
+                ek = relErr(dwk.download(), wdk), ev = relErr(dwv.download(), wdv), eo = relErr(dwo.download(), wdo);
+    std::printf("  %-40s  Y=%.2e dX=%.2e dWq=%.2e dWk=%.2e dWv=%.2e dWo=%.2e\n", name, ey, ex, eq, ek, ev, eo);
+    if (ey > tol || ex > tol || eq > tol || ek > tol || ev > tol || eo > tol) throw std::runtime_error(std::string(name) + " parity failed");
+    if (!layer.usedFlashAttention || layer.activePackCount != packs || layer.activeSegmentLength != T)
+        throw std::runtime_error("layer bookkeeping");
+}
+
+int main() {
+    try {
+        if (!sentinel_hip_device_available()) {
+            std::printf("  no HIP device\n");
+            return 2;
+        }
+        runCase("fp32 E64 H4 d16 T48", 64, 4, 4, 16, 48, 1, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
+        runCase("fp32 E64 H4 d16 T48 packs4", 64, 4, 4, 16, 48, 4, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
+        runCase("fp32 GQA E64 8q/2kv d8 T16 packs3", 64, 8, 2, 8, 16, 3, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
+        runCase("fp32 E96 H3 d32 T70 packs2", 96, 3, 3, 32, 70, 2, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
+        // MFMA arithmetic for the attention core (projections stay fp32), rotation fused into the conversion passes
+        runCase("bf16 E256 H4 d64 T128 packs2", 256, 4, 4, 64, 128, 2, SENTINEL_HIP_COMPUTE_BF16, 2e-2f);
+        runCase("fp16 GQA E256 4q/1kv d128 T200", 256, 4, 1, 128, 200, 1, SENTINEL_HIP_COMPUTE_F16, 2e-2f);
+        HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
+
+        // configurations this layer does not run are refused, not approximated
+        HostAttentionWeights host;
+        unsigned st = 9u;
+        host.embeddingDim = 32;
+        host.headCount = 2;
+        host.headDimension = 16;
+        host.maximumPositionCount = 32;
+        host.queryWeight = lcg(32 * 32, st, 0.1f);
+        host.keyWeight = host.queryWeight;
+        host.valueWeight = host.queryWeight;
+        host.outputWeight = host.queryWeight;
+        host.windowSize = 4;
+        HipCausalSelfAttention sparse = HipCausalSelfAttention::createFrom(host);
+        HipMatrix x, y;
+        x.ensureSize(32, 16);
+        x.fill(0.1f);
+        expectThrow("sliding window needs the dense path", [&] { sparse.forward(x, y); });
+        host.windowSize = 0;
+        HipCausalSelfAttention dense = HipCausalSelfAttention::createFrom(host);
+        expectThrow("columns not a multiple of the segment", [&] { dense.forward(x, y, 5); });
+        HipMatrix longer;
+        longer.ensureSize(32, 40);
+        longer.fill(0.1f);
+        expectThrow("sequence longer than the RoPE table", [&] { dense.forward(longer, y); });
+        HipMatrix dx, a, b, c, d;
+        HipCausalSelfAttention fresh = HipCausalSelfAttention::createFrom(host);
+        expectThrow("backward before forward", [&] { fresh.backward(x, dx, a, b, c, d); });
+        host.kvHeadCount = 3;
+        expectThrow("heads not divisible", [&] { HipCausalSelfAttention::createFrom(host); });
+        std::printf("  layer ok\n");
+        return 0;
+    } catch (const std::exception& ex) {
+        std::printf("  FAILED: %s\n", ex.what());
+        return 1;
+    }
+}

@@ -1,4 +1,4 @@
-"""The drop-in faces of the library on the GPU: the C++ shim (HipFlashAttention.hpp) and MFMA arithmetic on
+"""The drop-in faces of the library on the GPU: the C++ shims (HipFlashAttention.hpp, HipCausalSelfAttention.hpp) and MFMA arithmetic on
 Sentinel's own fp32 column layout (the adapter path), both through the C ABI."""
 import os
 import subprocess
@@ -21,6 +21,17 @@ def test_cpp_shim_parity_and_exceptions():
     print(proc.stdout, proc.stderr, flush=True)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "shim ok" in proc.stdout
+
+
+def test_cpp_attention_layer_parity_and_exceptions():
+    """HipCausalSelfAttention (projections + RoPE + flash attention + output projection, forward and backward) against
+    the oracle's layer; fp32 at 1e-4, MFMA arithmetic at 2e-2."""
+    exe = os.path.join(HERE, "cpp", "test_layer")
+    assert os.path.exists(exe), "tests/cpp/test_layer is not built: python -c 'import __graft_entry__ as g; g.build()'"
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=110)
+    print(proc.stdout, proc.stderr, flush=True)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "layer ok" in proc.stdout
 
 
 @pytest.mark.parametrize("compute", ["bf16", "fp16"])
