@@ -20,6 +20,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2516.6, "fp16": 2516.6, "fp32": 157.3}  # MI355X dense MFMA (256 CU x 2.4 GHz)
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
 # name: (B, Hq, Hkv, T, d, dtype, sigma_qk, description)
 CONFIGS = {
@@ -244,6 +245,53 @@ def columns_path(torch, name, steps, rope):
     return report
 
 
+def decode_path(torch, steps):
+    """The generation step's attention (one query column against the K/V cache, Sentinel's cache layout) against
+    the HBM roofline: algorithmic bytes = the used prefix of the K and V caches, 2 * kv_heads * d * length * 4,
+    read once, over the HIP-event time of the two launches (split scores / partial outputs, then the merge)."""
+    import sentinel_amd
+    lib = sentinel_amd.load_library()
+    report = {}
+    for label, (hq, hkv, d, length) in {
+        "gqa_32q_8kv_d128_L32768": (32, 8, 128, 32768),
+        "mha_32_d128_L4096": (32, 32, 128, 4096),
+        "gqa_32q_8kv_d128_L4096": (32, 8, 128, 4096),
+        "mha_16_d64_L16384": (16, 16, 64, 16384),
+        "mha_12_d64_L1024": (12, 12, 64, 1024),
+    }.items():
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(0x5E17 + length)
+        q = torch.randn(hq * d, 1, device="cuda", generator=gen)
+        k = torch.randn(hkv * d, length, device="cuda", generator=gen)
+        v = torch.randn(hkv * d, length, device="cuda", generator=gen)
+        out = torch.empty_like(q)
+        ws = torch.empty(lib.sentinel_hip_decode_workspace_bytes(hq, d, length) + 16, dtype=torch.uint8, device="cuda")
+        call = lambda: sentinel_amd.decode_attention(q, k, v, length, hq, d, kv_head_count=hkv, out=out, workspace=ws)
+        for _ in range(5):
+            call()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            call()
+        torch.cuda.synchronize()
+        wall_us = (time.perf_counter() - t0) / steps * 1e6
+        sentinel_amd.set_kernel_timing(True)
+        sentinel_amd.collect_kernel_timings()
+        for _ in range(steps):
+            call()
+        times = sentinel_amd.collect_kernel_timings()
+        sentinel_amd.set_kernel_timing(False)
+        partial_us = times["decode_partial"][0] / times["decode_partial"][1] * 1e3
+        merge_us = times["decode_merge"][0] / times["decode_merge"][1] * 1e3
+        cache_bytes = 2.0 * hkv * d * length * 4
+        achieved = cache_bytes / ((partial_us + merge_us) * 1e-6) / 1e9
+        report[label] = {"q_heads": hq, "kv_heads": hkv, "head_dim": d, "length": length, "cache_bytes": cache_bytes,
+                         "partial_us": partial_us, "merge_us": merge_us, "call_us_back_to_back": wall_us,
+                         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                      "frac": achieved / HBM_PEAK_GBS, "traffic": None}}
+    return report
+
+
 def rocminfo_gpu_clock_ghz():
     """Max Clock Freq. of the first gfx agent as printed by rocminfo (GHz), 0.0 if it cannot be read."""
     import re
@@ -271,6 +319,8 @@ def main():
     ap.add_argument("--columns-path", action="store_true",
                     help="also time the step through Sentinel's fp32 column layout (conversion passes, fused rotary "
                          "embedding) and report it under \"columns_path\"")
+    ap.add_argument("--decode-path", action="store_true",
+                    help="also time single-query attention against a K/V cache (generation) and report it under \"decode_path\"")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB -> 1 GiB elementwise copy kernel three times, so that a counter run "
                          "(FETCH_SIZE / WRITE_SIZE) of this command holds a kernel of known traffic to scale by")
@@ -373,6 +423,9 @@ def main():
         del w
         torch.cuda.empty_cache()
         line["columns_path"] = columns_path(torch, args.config, max(args.steps // 5, 3), rope=True)
+
+    if args.decode_path:
+        line["decode_path"] = decode_path(torch, max(args.steps, 20))
 
     if args.cpu_heads > 0:
         line["cpu_baseline"] = cpu_baseline(args.config, args.cpu_heads)

@@ -12,8 +12,12 @@
 // and the backward of each step. With 16-bit HipFlashAttention::computeType() the rotation rides on the layout
 // conversion (sentinel_hip_flash_fwd_rope / _bwd_rope) and query / key stay unrotated in the cache; with fp32
 // arithmetic they are rotated in place like the reference's.
-// Not built: the dense materialising fallback (sliding-window / global-token masks, flash disabled), KV-cache
-// prefill / decode; those configurations throw std::runtime_error instead of running something else.
+// Generation: HipKvCache mirrors CudaKvCache (Cuda/CudaKvCache.hpp:10-31), prefill / decode mirror
+// CudaCausalSelfAttention::prefill / decode (Cuda/CudaCausalSelfAttention.cu:549-575): the rotated K and V columns
+// are appended to the cache and the single query of a decode step attends to it with sentinel_hip_decode_attention
+// in place of attendCachedQuery's per-head copies and GEMMs (:318-341).
+// Not built: the dense materialising fallback (sliding-window / global-token masks, flash disabled); those
+// configurations throw std::runtime_error instead of running something else.
 // Link against libsentinel_hip_attn.so, rocBLAS and the HIP runtime.
 #ifndef SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
 #define SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
@@ -83,6 +87,58 @@ struct HostAttentionWeights {
     int globalTokenCount = 0;
 };
 
+/// append only device KV cache for one attention layer: key and value are embeddingDim x maximumPositionCount with
+/// a used prefix of `length` columns (class CudaKvCache, Cuda/CudaKvCache.hpp:10-31, Cuda/CudaKvCache.cu:9-43)
+class HipKvCache {
+public:
+    HipMatrix key;
+    HipMatrix value;
+    int length = 0;
+    int maximumPositionCount = 0;
+    int embeddingDim = 0;
+
+    /// allocate capacity and reset length to zero
+    void ensureCapacity(int embeddingDimension, int maximumPositions) {
+        if (embeddingDimension <= 0) throw std::invalid_argument("HipKvCache::ensureCapacity embeddingDim must be > 0");
+        if (maximumPositions <= 0) throw std::invalid_argument("HipKvCache::ensureCapacity maximumPositionCount must be > 0");
+        if (embeddingDim != embeddingDimension || maximumPositionCount != maximumPositions || key.empty() || value.empty()) {
+            key.ensureSize(static_cast<size_t>(embeddingDimension), static_cast<size_t>(maximumPositions));
+            value.ensureSize(static_cast<size_t>(embeddingDimension), static_cast<size_t>(maximumPositions));
+            throwIfHipFailed(hipMemsetAsync(key.buffer.deviceData, 0, key.byteCount(), HipFlashAttention::activeStream()), "HipKvCache zero key");
+            throwIfHipFailed(hipMemsetAsync(value.buffer.deviceData, 0, value.byteCount(), HipFlashAttention::activeStream()), "HipKvCache zero value");
+        }
+        embeddingDim = embeddingDimension;
+        maximumPositionCount = maximumPositions;
+        length = 0;
+    }
+
+    /// set length to zero keep capacity
+    void reset() { length = 0; }
+
+    /// append packed key and value columns embeddingDim x stepCount
+    void append(const HipMatrix& keyStep, const HipMatrix& valueStep) {
+        if (key.empty() || value.empty()) throw std::logic_error("HipKvCache::append capacity not allocated");
+        if (keyStep.empty() || valueStep.empty()) throw std::invalid_argument("HipKvCache::append empty step");
+        if (keyStep.rows != static_cast<size_t>(embeddingDim) || valueStep.rows != static_cast<size_t>(embeddingDim))
+            throw std::invalid_argument("HipKvCache::append embedding dim mismatch");
+        if (keyStep.cols != valueStep.cols) throw std::invalid_argument("HipKvCache::append step length mismatch");
+        const int stepCount = static_cast<int>(keyStep.cols);
+        if (length + stepCount > maximumPositionCount) throw std::invalid_argument("HipKvCache::append exceeds maximumPositionCount");
+        writeColumns(key, keyStep);
+        writeColumns(value, valueStep);
+        length += stepCount;
+    }
+
+private:
+    // the step's columns land behind the used prefix of every row: a strided 2-D copy
+    void writeColumns(HipMatrix& cache, const HipMatrix& step) const {
+        throwIfHipFailed(hipMemcpy2DAsync(cache.buffer.deviceData + length, cache.cols * sizeof(float), step.buffer.deviceData,
+                                          step.cols * sizeof(float), step.cols * sizeof(float), step.rows,
+                                          hipMemcpyDeviceToDevice, HipFlashAttention::activeStream()),
+                         "HipKvCache::append copy");
+    }
+};
+
 class HipCausalSelfAttention {
 public:
     HipMatrix queryWeight, keyWeight, valueWeight, outputWeight;
@@ -102,6 +158,7 @@ public:
     HipMatrix query, key, value, attended, output;
     HipMatrix inputCache, attendedGradient, queryGradient, keyGradient, valueGradient;
     HipMatrix flashLogSumExp, flashDelta;
+    HipDeviceBuffer decodeWorkspace;
 
     /// upload weights and build the RoPE tables the way RotaryEmbedding does (Layers/RotaryEmbedding.cpp:8-29)
     void uploadFrom(const HostAttentionWeights& host) {
@@ -219,7 +276,70 @@ public:
         HipGemm::multiplyInto(valueWeight, valueGradient, inputGradient, true, false, true);
     }
 
+    /// reset cache then run full sequence attention and append rotated KV
+    void prefill(const HipMatrix& input, HipKvCache& cache, HipMatrix& out) {
+        const char* op = "HipCausalSelfAttention::prefill";
+        if (input.empty()) throw std::invalid_argument(std::string(op) + " empty input");
+        if (queryWeight.empty()) throw std::logic_error(std::string(op) + " weights not uploaded");
+        if (queryWeight.cols != input.rows) throw std::invalid_argument(std::string(op) + " embedding dim mismatch");
+        if (static_cast<int>(input.cols) > maximumPositionCount)
+            throw std::invalid_argument(std::string(op) + " sequence longer than maximumPositionCount");
+        if (!canUseFlashAttention(static_cast<int>(input.cols)))
+            throw std::runtime_error(std::string(op) + " needs the dense attention path (sparse window or flash disabled), which is not built");
+        cache.ensureCapacity(static_cast<int>(keyWeight.rows), maximumPositionCount);
+        projectAndRotate(input, 0);
+        cache.append(key, value);
+        const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
+        HipFlashAttention::forwardMultiHead(query, key, value, attended, flashLogSumExp, headCount, headDimension, scale, true, 0,
+                                            static_cast<int>(input.cols), 1, kvHeadCount);
+        HipGemm::multiplyInto(outputWeight, attended, out);
+    }
+
+    /// single token attention against append only KV cache
+    void decode(const HipMatrix& input, HipKvCache& cache, HipMatrix& out) {
+        const char* op = "HipCausalSelfAttention::decode";
+        if (input.empty()) throw std::invalid_argument(std::string(op) + " empty input");
+        if (input.cols != 1) throw std::invalid_argument(std::string(op) + " expects a single token column");
+        if (queryWeight.empty()) throw std::logic_error(std::string(op) + " weights not uploaded");
+        if (queryWeight.cols != input.rows) throw std::invalid_argument(std::string(op) + " embedding dim mismatch");
+        if (cache.key.empty() || cache.value.empty()) throw std::logic_error(std::string(op) + " cache not allocated");
+        if (cache.length >= cache.maximumPositionCount) throw std::invalid_argument(std::string(op) + " cache full");
+        if (cache.length >= maximumPositionCount) throw std::invalid_argument(std::string(op) + " position exceeds RoPE table");
+        projectAndRotate(input, cache.length);
+        cache.append(key, value);
+        attendCachedQuery(cache, out);
+    }
+
 private:
+    // Q, K, V projections of the input columns, Q and K rotated in place for positions offset, offset + 1, ...
+    // (CudaCausalSelfAttention::projectAndRotate, Cuda/CudaCausalSelfAttention.cu:181-208)
+    void projectAndRotate(const HipMatrix& input, int positionOffset) {
+        HipGemm::multiplyInto(queryWeight, input, query);
+        HipGemm::multiplyInto(keyWeight, input, key);
+        HipGemm::multiplyInto(valueWeight, input, value);
+        HipOps::rotaryRotateInPlace(query, headCount, headDimension, pairCount, cosTable, sinTable, positionOffset);
+        HipOps::rotaryRotateInPlace(key, kvHeadCount, headDimension, pairCount, cosTable, sinTable, positionOffset);
+    }
+
+    void attendCachedQuery(const HipKvCache& cache, HipMatrix& out) {
+        const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
+        attended.ensureSize(query.rows, 1);
+        const size_t need = sentinel_hip_decode_workspace_bytes(headCount, headDimension, cache.length);
+        decodeWorkspace.ensureCapacity(need);
+        const int code = sentinel_hip_decode_attention(query.buffer.deviceData, cache.key.buffer.deviceData,
+                                                       cache.value.buffer.deviceData, attended.buffer.deviceData, headCount,
+                                                       kvHeadCount, headDimension, cache.maximumPositionCount, cache.length, scale,
+                                                       windowSize, globalTokenCount, decodeWorkspace.deviceData, need,
+                                                       HipFlashAttention::activeStream());
+        if (code != SENTINEL_HIP_OK) {
+            std::string detail = sentinel_hip_last_error();
+            if (detail.empty()) detail = sentinel_hip_strerror(code);
+            if (code == SENTINEL_HIP_RUNTIME) throw std::runtime_error(detail);
+            throw std::invalid_argument(detail);
+        }
+        HipGemm::multiplyInto(outputWeight, attended, out);
+    }
+
     // the rotation rides on the fp32 <-> 16-bit conversion when there is one
     bool fusedRotation() const {
         const int compute = HipFlashAttention::computeType();

@@ -139,6 +139,24 @@ SENTINEL_HIP_API int sentinel_hip_flash_bwd_rope(const void* q, const void* k, c
                                 int column_start, int seq_len, int pack_count, float scale, int causal, void* workspace,
                                 size_t workspace_bytes, void* stream);
 
+/*
+ * Generation step: attention of ONE query position (the newest token, rows q_heads*head_dim of `query`, already
+ * rotated) against the first `length` positions of an append-only K/V cache in Sentinel's layout: fp32
+ * [(kv_head*head_dim + dim), position] with cache_stride positions per row (CudaKvCache::key / ::value,
+ * Cuda/CudaKvCache.hpp:9-29; the new token's K/V are appended before the call, so length includes it).
+ * out = q_heads*head_dim floats, the attended vector before the output projection.
+ * Replaces the per-head loop of CudaCausalSelfAttention::attendCachedQuery
+ * (Cuda/CudaCausalSelfAttention.cu:318-341; extractHead x3, GEMM, scale, mask, softmax, GEMM, writeHead per head)
+ * with two launches that read the cache once; grouped-query heads share the reads. window_size /
+ * global_token_count are the layer's sparse-mask parameters: only the full causal case (window_size <= 0 or
+ * >= length) is built, anything else returns SENTINEL_HIP_UNSUPPORTED. Workspace: sentinel_hip_decode_workspace_bytes.
+ */
+SENTINEL_HIP_API size_t sentinel_hip_decode_workspace_bytes(int q_heads, int head_dim, int length);
+SENTINEL_HIP_API int sentinel_hip_decode_attention(const float* query, const float* key_cache, const float* value_cache, float* out,
+                                  int q_heads, int kv_heads, int head_dim, int cache_stride, int length, float scale,
+                                  int window_size, int global_token_count, void* workspace, size_t workspace_bytes,
+                                  void* stream);
+
 /* Largest head_dim any kernel here accepts (the CUDA path's CudaFlashAttention::maxHeadDimension is 64). */
 SENTINEL_HIP_API int sentinel_hip_flash_max_head_dim(void);
 

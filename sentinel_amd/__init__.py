@@ -3,6 +3,7 @@ from .flash_attention import (  # noqa: F401
     HipFlashAttention,
     HipOps,
     collect_kernel_timings,
+    decode_attention,
     flash_attention_backward,
     flash_attention_forward,
     library_path,

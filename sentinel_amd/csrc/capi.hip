@@ -420,3 +420,38 @@ extern "C" int sentinel_hip_rope_rotate(float* tensor, int heads, int head_dim, 
     if (err != hipSuccess) return fail_hip("rope rotate launch", err);
     return SENTINEL_HIP_OK;
 }
+
+extern "C" size_t sentinel_hip_decode_workspace_bytes(int q_heads, int head_dim, int length) {
+    if (q_heads <= 0 || head_dim <= 0 || length <= 0) return 0;
+    return align_up(decode_workspace_bytes(q_heads, head_dim, length));
+}
+
+extern "C" int sentinel_hip_decode_attention(const float* query, const float* key_cache, const float* value_cache, float* out,
+                                             int q_heads, int kv_heads, int head_dim, int cache_stride, int length,
+                                             float scale, int window_size, int global_token_count, void* workspace,
+                                             size_t workspace_bytes, void* stream_ptr) {
+    const char* op = "sentinel_hip_decode_attention";
+    if (!query || !key_cache || !value_cache || !out) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
+    if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s invalid head geometry", op);
+    if (q_heads % kv_heads != 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s headCount must be divisible by kvHeadCount", op);
+    if (head_dim > sentinel_hip_flash_max_head_dim()) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s headDim exceeds maxHeadDimension", op);
+    if (length <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s cache is empty", op);
+    if (length > cache_stride) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s cache length exceeds its capacity", op);
+    if (!(scale > 0.0f) || !std::isfinite(scale)) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s scale must be positive and finite", op);
+    (void)global_token_count;
+    if (window_size > 0 && window_size < length)
+        return fail(SENTINEL_HIP_UNSUPPORTED, "%s sliding-window masks are not built (window %d < cache length %d)", op, window_size, length);
+    const int group = q_heads / kv_heads;
+    if (group != 1 && group != 2 && group != 4 && group != 8)
+        return fail(SENTINEL_HIP_UNSUPPORTED, "%s query heads per K/V head must be 1, 2, 4 or 8 (got %d)", op, group);
+    if (head_dim % 8 != 0) return fail(SENTINEL_HIP_UNSUPPORTED, "%s head_dim must be a multiple of 8", op);
+    const size_t need = sentinel_hip_decode_workspace_bytes(q_heads, head_dim, length);
+    if (!workspace || workspace_bytes < need || misaligned(workspace))
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s needs %zu bytes of 16-byte aligned workspace", op, need);
+    if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
+    const hipError_t err = launch_decode_attention(query, key_cache, value_cache, out, q_heads, kv_heads, head_dim,
+                                                   cache_stride, length, scale, static_cast<float*>(workspace),
+                                                   static_cast<hipStream_t>(stream_ptr));
+    if (err != hipSuccess) return fail_hip("decode attention launch", err);
+    return SENTINEL_HIP_OK;
+}

@@ -68,6 +68,11 @@ hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int he
                                   int seq_len, int packs, RopeTables rope, hipStream_t stream);
 hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,
                                   int seq_len, int packs, RopeTables inverse_rope, hipStream_t stream);
+// single-query attention against the K/V cache (fp32 column layout, `stride` positions per row, `length` used)
+size_t decode_workspace_bytes(int q_heads, int head_dim, int length);
+hipError_t launch_decode_attention(const float* query, const float* key_cache, const float* value_cache, float* out,
+                                   int q_heads, int kv_heads, int head_dim, int stride, int length, float scale,
+                                   float* workspace, hipStream_t stream);
 // in-place rotation of fp32 column-layout rows (tensor already advanced to the first column)
 hipError_t launch_rope_rotate_f32(float* tensor, int heads, int head_dim, int stride_columns, int columns,
                                   int position_offset, int segment_length, const float* cos, const float* sin, bool inverse,

@@ -57,6 +57,10 @@ def load_library():
     lib.sentinel_hip_flash_bwd_rope.restype = i
     lib.sentinel_hip_rope_rotate.argtypes = [vp] + [i] * 7 + [vp, vp, i, i, vp]
     lib.sentinel_hip_rope_rotate.restype = i
+    lib.sentinel_hip_decode_workspace_bytes.argtypes = [i] * 3
+    lib.sentinel_hip_decode_workspace_bytes.restype = sz
+    lib.sentinel_hip_decode_attention.argtypes = [vp] * 4 + [i] * 5 + [f, i, i, vp, sz, vp]
+    lib.sentinel_hip_decode_attention.restype = i
     lib.sentinel_hip_flash_workspace_bytes.argtypes = [i] * 9
     lib.sentinel_hip_flash_workspace_bytes.restype = sz
     lib.sentinel_hip_flash_max_head_dim.restype = i
@@ -280,6 +284,34 @@ class HipFlashAttention:
             raise ValueError(f"{name} sequenceLength mismatch")
         if not load_library().sentinel_hip_device_available():
             raise RuntimeError(f"{name} no HIP device")
+
+
+def decode_attention(query, key_cache, value_cache, length, head_count, head_dimension, *, kv_head_count=None, scale=None,
+                     window_size=0, global_token_count=0, out=None, workspace=None, stream=None):
+    """Attention of the newest token against the first `length` positions of the K/V cache
+    (CudaCausalSelfAttention::attendCachedQuery without the output projection).
+
+    query: fp32 [head_count*head_dimension, 1]; caches: fp32 [kv_heads*head_dimension, capacity]. Returns out [rows, 1]."""
+    lib = load_library()
+    kv_heads = head_count if kv_head_count in (None, 0) else kv_head_count
+    for t in (query, key_cache, value_cache):
+        if t is None or t.dim() != 2 or t.numel() == 0:
+            raise ValueError("decode_attention empty input")
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise ValueError("decode_attention expects contiguous fp32 matrices")
+    if query.shape != (head_count * head_dimension, 1):
+        raise ValueError("decode_attention expects a single token column")
+    if key_cache.shape[0] != kv_heads * head_dimension or value_cache.shape != key_cache.shape:
+        raise ValueError("decode_attention key/value rows mismatch")
+    scale = 1.0 / math.sqrt(head_dimension) if scale is None else float(scale)
+    out = _ensure_size(out, head_count * head_dimension, 1, query)
+    need = lib.sentinel_hip_decode_workspace_bytes(head_count, head_dimension, max(int(length), 1))
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=query.device)
+    _check(lib.sentinel_hip_decode_attention(_ptr(query), _ptr(key_cache), _ptr(value_cache), _ptr(out), head_count, kv_heads,
+                                             head_dimension, int(key_cache.shape[1]), int(length), scale, int(window_size),
+                                             int(global_token_count), _ptr(workspace), need, _stream_handle(stream)))
+    return out
 
 
 def _bhtd_geometry(q, k, v):

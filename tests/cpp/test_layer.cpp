@@ -1,5 +1,5 @@
 // GPU test of the C++ attention layer (include/sentinel_hip/HipCausalSelfAttention.hpp) against the CPU oracle's
-// layer, on the shapes of the reference's own device smoke tests (CudaCausalSelfAttention::runFlashParitySmokeDemo:
+// layer (training step and prefill / decode generation), on the shapes of the reference's own device smoke tests (CudaCausalSelfAttention::runFlashParitySmokeDemo:
 // E=64, H=4, T=48; runGqaCudaSmokeDemo: grouped heads) plus packed batches and head_dim 64 / 128 with MFMA arithmetic.
 // Test infrastructure: the oracle is linked here only as the checker.
 #include "../../include/sentinel_hip/HipCausalSelfAttention.hpp"
@@ -98,6 +98,60 @@ static void runCase(const char* name, int e, int heads, int kvHeads, int d, int 
         throw std::runtime_error("layer bookkeeping");
 }
 
+// Generation: prefill `prompt` columns, then decode the rest one token at a time. Step t must reproduce column t of
+// the oracle's full forward over columns 0..t (causal attention: earlier columns do not depend on later ones, so
+// one oracle call over all columns gives every step's answer).
+static void runGeneration(const char* name, int e, int heads, int kvHeads, int d, int prompt, int total, int compute, float tol) {
+    const int qRows = heads * d, kvRows = kvHeads * d;
+    unsigned state = 4711u + static_cast<unsigned>(e + total);
+    const float bound = 1.0f / std::sqrt(static_cast<float>(e));
+    HostAttentionWeights host;
+    host.queryWeight = lcg(static_cast<size_t>(qRows) * e, state, bound);
+    host.keyWeight = lcg(static_cast<size_t>(kvRows) * e, state, bound);
+    host.valueWeight = lcg(static_cast<size_t>(kvRows) * e, state, bound);
+    host.outputWeight = lcg(static_cast<size_t>(e) * qRows, state, bound);
+    host.embeddingDim = e;
+    host.headCount = heads;
+    host.kvHeadCount = kvHeads;
+    host.headDimension = d;
+    host.maximumPositionCount = total;
+    auto hx = lcg(static_cast<size_t>(e) * total, state, 1.0f);
+    std::vector<float> want(hx.size());
+    if (sentinel_oracle_layer(hx.data(), host.queryWeight.data(), host.keyWeight.data(), host.valueWeight.data(),
+                              host.outputWeight.data(), nullptr, want.data(), nullptr, nullptr, nullptr, nullptr, nullptr, e, heads,
+                              kvHeads, d, total, host.ropeBase, host.maximumPositionCount) != 0)
+        throw std::runtime_error("oracle layer failed");
+
+    HipFlashAttention::computeType() = compute;
+    HipCausalSelfAttention layer = HipCausalSelfAttention::createFrom(host);
+    HipKvCache cache;
+    auto columns = [&](const std::vector<float>& m, int c0, int count) {
+        std::vector<float> out(static_cast<size_t>(e) * count);
+        for (int r = 0; r < e; ++r)
+            for (int c = 0; c < count; ++c) out[static_cast<size_t>(r) * count + c] = m[static_cast<size_t>(r) * total + c0 + c];
+        return out;
+    };
+    HipMatrix x, y;
+    x.upload(columns(hx, 0, prompt), e, prompt);
+    layer.prefill(x, cache, y);
+    float worst = relErr(y.download(), columns(want, 0, prompt));
+    if (cache.length != prompt) throw std::runtime_error("prefill did not fill the cache");
+    for (int t = prompt; t < total; ++t) {
+        x.upload(columns(hx, t, 1), e, 1);
+        layer.decode(x, cache, y);
+        worst = std::max(worst, relErr(y.download(), columns(want, t, 1)));
+    }
+    std::printf("  %-40s  worst step error %.2e\n", name, worst);
+    if (worst > tol) throw std::runtime_error(std::string(name) + " generation parity failed");
+    if (cache.length != total) throw std::runtime_error("decode did not extend the cache");
+    x.upload(columns(hx, 0, 1), e, 1);
+    expectThrow("cache full", [&] { layer.decode(x, cache, y); });
+    // prefill resets the cache
+    x.upload(columns(hx, 0, prompt), e, prompt);
+    layer.prefill(x, cache, y);
+    if (cache.length != prompt) throw std::runtime_error("prefill did not reset the cache");
+}
+
 int main() {
     try {
         if (!sentinel_hip_device_available()) {
@@ -111,6 +165,12 @@ int main() {
         // MFMA arithmetic for the attention core (projections stay fp32), rotation fused into the conversion passes
         runCase("bf16 E256 H4 d64 T128 packs2", 256, 4, 4, 64, 128, 2, SENTINEL_HIP_COMPUTE_BF16, 2e-2f);
         runCase("fp16 GQA E256 4q/1kv d128 T200", 256, 4, 1, 128, 200, 1, SENTINEL_HIP_COMPUTE_F16, 2e-2f);
+        HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
+        // the shapes of runKvCacheSmokeDemo (E=64, H=4, T=32 of 64 positions), grouped heads, a cache of several chunks
+        runGeneration("generate fp32 E64 H4 d16 32+32", 64, 4, 4, 16, 32, 64, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
+        runGeneration("generate fp32 GQA 8q/2kv d8 5+20", 64, 8, 2, 8, 5, 25, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
+        runGeneration("generate fp32 E128 H2 d64 1+300", 128, 2, 2, 64, 1, 301, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
+        runGeneration("generate bf16 prefill GQA 4q/1kv d128", 256, 4, 1, 128, 130, 140, SENTINEL_HIP_COMPUTE_BF16, 2e-2f);
         HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
 
         // configurations this layer does not run are refused, not approximated
