@@ -38,7 +38,7 @@ Matrix selection(int rows, int cols, int colOffset) {
 
 void runLayer(const float* q, const float* k, const float* v, float* out, float* lse, const float* dOut, float* dq,
               float* dk, float* dv, int qHeads, int kvHeads, int d, size_t stride, size_t col0, int t, int qHead0,
-              int kvHead0, bool accumulateKv) {
+              int kvHead0, bool accumulateKv, int windowSize = 0, int globalTokenCount = 0, bool preferSparse = true) {
     const int qRows = qHeads * d;
     const int kvRows = kvHeads * d;
     const int embed = qRows + 2 * kvRows;
@@ -48,8 +48,9 @@ void runLayer(const float* q, const float* k, const float* v, float* out, float*
     std::fill(rope.sinTable.begin(), rope.sinTable.end(), 0.0f);
 
     CausalSelfAttention layer(selection(qRows, embed, 0), selection(kvRows, embed, qRows),
-                              selection(kvRows, embed, qRows + kvRows), selection(qRows, qRows, 0), rope, qHeads, t, 0,
-                              kvHeads);
+                              selection(kvRows, embed, qRows + kvRows), selection(qRows, qRows, 0), rope, qHeads,
+                              windowSize > 0 ? windowSize : t, globalTokenCount, kvHeads);
+    layer.preferSparseCompute = preferSparse;
 
     Matrix x(static_cast<size_t>(embed), static_cast<size_t>(t), 0.0f);
     for (int r = 0; r < qRows; ++r)
@@ -132,6 +133,26 @@ extern "C" int sentinel_ref_attention(const float* q, const float* k, const floa
             for (int h = 0; h < qHeads; ++h)
                 runLayer(q, k, v, out, lse, d_out, dq, dk, dv, 1, 1, headDim, stride, col0, seqLen, h, h / group, true);
         }
+        return 0;
+    } catch (const std::exception&) {
+        return -2;
+    }
+}
+
+/*
+ * The layer's sparse mask (windowSize, globalTokenCount; Layers/CausalSelfAttention.cpp:95-120), one layer call
+ * per pack with all heads.  preferSparse = 0: dense masked path; 1: the sparse-compute path (:128-168).
+ */
+extern "C" int sentinel_ref_attention_sparse(const float* q, const float* k, const float* v, float* out, float* lse,
+                                             const float* d_out, float* dq, float* dk, float* dv, int qHeads, int kvHeads,
+                                             int headDim, int strideColumns, int colStart, int seqLen, int packCount,
+                                             int windowSize, int globalTokenCount, int preferSparse) {
+    try {
+        if (qHeads <= 0 || kvHeads <= 0 || qHeads % kvHeads != 0) return -1;
+        for (int pack = 0; pack < packCount; ++pack)
+            runLayer(q, k, v, out, lse, d_out, dq, dk, dv, qHeads, kvHeads, headDim, static_cast<size_t>(strideColumns),
+                     static_cast<size_t>(colStart) + static_cast<size_t>(pack) * seqLen, seqLen, 0, 0, false, windowSize,
+                     globalTokenCount, preferSparse != 0);
         return 0;
     } catch (const std::exception&) {
         return -2;

@@ -176,7 +176,17 @@ struct Geometry {
     size_t stride, t;
     float scale;
     bool causal;
+    int window = 0;        // sliding window (<= 0: none)
+    int globalTokens = 0;  // keys before this index are visible to every later query
 };
+
+// CausalSelfAttention::allowsKey (Layers/CausalSelfAttention.cpp:95-100)
+bool allowsKey(long long query, long long key, int window, int globalTokens) {
+    if (key > query) return false;
+    if (key < globalTokens) return true;
+    if (window <= 0) return true;
+    return key >= query - window + 1;
+}
 
 void onePack(const Geometry& g, size_t col0, const float* q, const float* k, const float* v, float* out, float* lse,
              const float* dOut, float* dq, float* dk, float* dv, Scratch& s) {
@@ -211,9 +221,13 @@ void onePack(const Geometry& g, size_t col0, const float* q, const float* k, con
         // scores[key][query] = scale * sum_dim K[dim][key] Q[dim][query], then mask (CausalSelfAttention.cpp:122-126)
         gemm(s.kHead.data(), d, t, s.qHead.data(), d, t, s.scores.data(), true, false, s);
         for (size_t i = 0; i < t * t; ++i) s.scores[i] *= g.scale;
+        // applyAttentionMaskInPlace (CausalSelfAttention.cpp:109-120): the dense masked path, which the reference's
+        // sparse-compute path (:128-168) reproduces up to summation order
         if (g.causal)
             for (size_t key = 0; key < t; ++key)
-                for (size_t query = 0; query < key && query < t; ++query) s.scores[key * t + query] = -1e9f;
+                for (size_t query = 0; query < t; ++query)
+                    if (!allowsKey(static_cast<long long>(query), static_cast<long long>(key), g.window, g.globalTokens))
+                        s.scores[key * t + query] = -1e9f;
 
         softmaxColumns(s.scores.data(), s.probs.data(), t, t);
 
@@ -248,7 +262,9 @@ void onePack(const Geometry& g, size_t col0, const float* q, const float* k, con
         }
         if (g.causal)  // CausalSelfAttention.cpp:338-343
             for (size_t key = 0; key < t; ++key)
-                for (size_t query = 0; query < key && query < t; ++query) s.dScores[key * t + query] = 0.0f;
+                for (size_t query = 0; query < t; ++query)
+                    if (!allowsKey(static_cast<long long>(query), static_cast<long long>(key), g.window, g.globalTokens))
+                        s.dScores[key * t + query] = 0.0f;
         for (size_t i = 0; i < t * t; ++i) s.dScores[i] *= g.scale;
         // dQ = K dS ; dK = Q dS^T (CausalSelfAttention.cpp:346-347)
         gemm(s.kHead.data(), d, t, s.dScores.data(), t, t, s.dqHead.data(), false, false, s);
@@ -262,10 +278,11 @@ void onePack(const Geometry& g, size_t col0, const float* q, const float* k, con
 
 }  // namespace
 
-extern "C" int sentinel_oracle_attention(const float* q, const float* k, const float* v, float* out, float* lse,
-                                         const float* d_out, float* dq, float* dk, float* dv, int qHeads, int kvHeads,
-                                         int headDim, int strideColumns, int colStart, int seqLen, int packCount,
-                                         float scale, int causal, int packParallel) {
+extern "C" int sentinel_oracle_attention_sparse(const float* q, const float* k, const float* v, float* out, float* lse,
+                                                const float* d_out, float* dq, float* dk, float* dv, int qHeads,
+                                                int kvHeads, int headDim, int strideColumns, int colStart, int seqLen,
+                                                int packCount, float scale, int causal, int packParallel, int windowSize,
+                                                int globalTokenCount) {
     if (!q || !k || !v || !out) return -1;
     if (qHeads <= 0 || kvHeads <= 0 || headDim <= 0 || qHeads % kvHeads != 0) return -1;
     if (seqLen <= 0 || packCount <= 0 || colStart < 0) return -1;
@@ -273,7 +290,10 @@ extern "C" int sentinel_oracle_attention(const float* q, const float* k, const f
     const bool wantBackward = d_out != nullptr;
     if (wantBackward != (dq != nullptr) || wantBackward != (dk != nullptr) || wantBackward != (dv != nullptr)) return -1;
 
-    Geometry g{qHeads, kvHeads, headDim, static_cast<size_t>(strideColumns), static_cast<size_t>(seqLen), scale, causal != 0};
+    if (globalTokenCount < 0) return -1;
+    if (!causal && (windowSize > 0 || globalTokenCount > 0)) return -1;  // the sparse mask refines the causal one
+    Geometry g{qHeads, kvHeads, headDim, static_cast<size_t>(strideColumns), static_cast<size_t>(seqLen), scale, causal != 0,
+               windowSize, globalTokenCount};
 
     if (packParallel && packCount > 1) {
 #if defined(_OPENMP)
@@ -295,6 +315,14 @@ extern "C" int sentinel_oracle_attention(const float* q, const float* k, const f
         onePack(g, static_cast<size_t>(colStart) + static_cast<size_t>(pack) * g.t, q, k, v, out, lse, d_out, dq, dk, dv,
                 scratch);
     return 0;
+}
+
+extern "C" int sentinel_oracle_attention(const float* q, const float* k, const float* v, float* out, float* lse,
+                                         const float* d_out, float* dq, float* dk, float* dv, int qHeads, int kvHeads,
+                                         int headDim, int strideColumns, int colStart, int seqLen, int packCount,
+                                         float scale, int causal, int packParallel) {
+    return sentinel_oracle_attention_sparse(q, k, v, out, lse, d_out, dq, dk, dv, qHeads, kvHeads, headDim, strideColumns,
+                                            colStart, seqLen, packCount, scale, causal, packParallel, 0, 0);
 }
 
 extern "C" int sentinel_oracle_delta(const float* out, const float* d_out, float* delta, int qHeads, int headDim,
@@ -380,11 +408,13 @@ extern "C" int sentinel_oracle_rope_rotate(float* tensor, int heads, int headDim
     return 0;
 }
 
-// Layers/CausalSelfAttention.cpp:212-264 (forward) and :266-368 (backward), full causal mask
-extern "C" int sentinel_oracle_layer(const float* x, const float* wq, const float* wk, const float* wv, const float* wo,
-                                     const float* d_y, float* y, float* d_x, float* d_wq, float* d_wk, float* d_wv,
-                                     float* d_wo, int embeddingDim, int qHeads, int kvHeads, int headDim, int seqLen,
-                                     float ropeBase, int ropePositions) {
+// Layers/CausalSelfAttention.cpp:212-264 (forward) and :266-368 (backward); windowSize <= 0 and globalTokenCount 0
+// give the full causal mask
+extern "C" int sentinel_oracle_layer_sparse(const float* x, const float* wq, const float* wk, const float* wv,
+                                            const float* wo, const float* d_y, float* y, float* d_x, float* d_wq,
+                                            float* d_wk, float* d_wv, float* d_wo, int embeddingDim, int qHeads, int kvHeads,
+                                            int headDim, int seqLen, float ropeBase, int ropePositions, int windowSize,
+                                            int globalTokenCount) {
     if (!x || !wq || !wk || !wv || !wo || !y) return -1;
     if (embeddingDim <= 0 || qHeads <= 0 || kvHeads <= 0 || qHeads % kvHeads != 0 || headDim <= 0 || headDim % 2 != 0) return -1;
     if (seqLen <= 0 || seqLen > ropePositions) return -1;
@@ -402,22 +432,23 @@ extern "C" int sentinel_oracle_layer(const float* x, const float* wq, const floa
     sentinel_oracle_rope_rotate(k.data(), kvHeads, headDim, t, 0, t, 0, 0, cosT.data(), sinT.data(), ropePositions, 0);
     const float scale = 1.0f / std::sqrt(static_cast<float>(headDim));
     if (!wantBackward) {
-        if (sentinel_oracle_attention(q.data(), k.data(), v.data(), a.data(), nullptr, nullptr, nullptr, nullptr, nullptr,
-                                      qHeads, kvHeads, headDim, t, 0, t, 1, scale, 1, 0) != 0)
+        if (sentinel_oracle_attention_sparse(q.data(), k.data(), v.data(), a.data(), nullptr, nullptr, nullptr, nullptr, nullptr,
+                                             qHeads, kvHeads, headDim, t, 0, t, 1, scale, 1, 0, windowSize, globalTokenCount) != 0)
             return -1;
         sentinel_oracle_gemm(wo, e, qRows, a.data(), qRows, t, y, 0, 0);
         return 0;
     }
     std::vector<float> dA(q.size()), dq(q.size()), dk(k.size()), dv(k.size()), temp(static_cast<size_t>(e) * t);
     // forward once for A (and Y), then the backward from dA = Wo^T dY
-    if (sentinel_oracle_attention(q.data(), k.data(), v.data(), a.data(), nullptr, nullptr, nullptr, nullptr, nullptr, qHeads,
-                                  kvHeads, headDim, t, 0, t, 1, scale, 1, 0) != 0)
+    if (sentinel_oracle_attention_sparse(q.data(), k.data(), v.data(), a.data(), nullptr, nullptr, nullptr, nullptr, nullptr,
+                                         qHeads, kvHeads, headDim, t, 0, t, 1, scale, 1, 0, windowSize, globalTokenCount) != 0)
         return -1;
     sentinel_oracle_gemm(wo, e, qRows, a.data(), qRows, t, y, 0, 0);
     sentinel_oracle_gemm(d_y, e, t, a.data(), qRows, t, d_wo, 0, 1);
     sentinel_oracle_gemm(wo, e, qRows, d_y, e, t, dA.data(), 1, 0);
-    if (sentinel_oracle_attention(q.data(), k.data(), v.data(), a.data(), nullptr, dA.data(), dq.data(), dk.data(), dv.data(),
-                                  qHeads, kvHeads, headDim, t, 0, t, 1, scale, 1, 0) != 0)
+    if (sentinel_oracle_attention_sparse(q.data(), k.data(), v.data(), a.data(), nullptr, dA.data(), dq.data(), dk.data(),
+                                         dv.data(), qHeads, kvHeads, headDim, t, 0, t, 1, scale, 1, 0, windowSize,
+                                         globalTokenCount) != 0)
         return -1;
     sentinel_oracle_rope_rotate(dq.data(), qHeads, headDim, t, 0, t, 0, 0, cosT.data(), sinT.data(), ropePositions, 1);
     sentinel_oracle_rope_rotate(dk.data(), kvHeads, headDim, t, 0, t, 0, 0, cosT.data(), sinT.data(), ropePositions, 1);
@@ -430,6 +461,14 @@ extern "C" int sentinel_oracle_layer(const float* x, const float* wq, const floa
     sentinel_oracle_gemm(wv, kvRows, e, dv.data(), kvRows, t, temp.data(), 1, 0);
     for (size_t i = 0; i < temp.size(); ++i) d_x[i] += temp[i];
     return 0;
+}
+
+extern "C" int sentinel_oracle_layer(const float* x, const float* wq, const float* wk, const float* wv, const float* wo,
+                                     const float* d_y, float* y, float* d_x, float* d_wq, float* d_wk, float* d_wv,
+                                     float* d_wo, int embeddingDim, int qHeads, int kvHeads, int headDim, int seqLen,
+                                     float ropeBase, int ropePositions) {
+    return sentinel_oracle_layer_sparse(x, wq, wk, wv, wo, d_y, y, d_x, d_wq, d_wk, d_wv, d_wo, embeddingDim, qHeads, kvHeads,
+                                        headDim, seqLen, ropeBase, ropePositions, 0, 0);
 }
 
 extern "C" int sentinel_oracle_max_threads(void) {

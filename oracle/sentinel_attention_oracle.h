@@ -43,6 +43,24 @@ int sentinel_oracle_attention(const float* q, const float* k, const float* v,
                               int strideColumns, int colStart, int seqLen, int packCount,
                               float scale, int causal, int packParallel);
 
+/*
+ * The same with Sentinel's sparse mask on top of the causal one (CausalSelfAttention::allowsKey,
+ * Layers/CausalSelfAttention.cpp:95-100): key <= query and (key < globalTokenCount or windowSize <= 0 or
+ * key >= query - windowSize + 1).  Restates the dense masked path (applyAttentionMaskInPlace :109-120, score
+ * gradients zeroed :338-343); the reference's sparse-compute path (:128-168, :296-330) skips the forbidden pairs
+ * instead and agrees up to summation order.  windowSize = 0, globalTokenCount = 0 is sentinel_oracle_attention.
+ * Pinned bit-exactly against the reference's compiled layer with preferSparseCompute = false, to rounding with
+ * preferSparseCompute = true, and against a float64 masked softmax (tests/test_oracle_sparse.py).
+ * Returns -1 for a window / global tokens without the causal flag.
+ */
+int sentinel_oracle_attention_sparse(const float* q, const float* k, const float* v,
+                                     float* out, float* lse,
+                                     const float* d_out, float* dq, float* dk, float* dv,
+                                     int qHeads, int kvHeads, int headDim,
+                                     int strideColumns, int colStart, int seqLen, int packCount,
+                                     float scale, int causal, int packParallel,
+                                     int windowSize, int globalTokenCount);
+
 /* D[head][column] = sum_dim out * d_out (Cuda/CudaFlashAttention.cu:576-596). */
 int sentinel_oracle_delta(const float* out, const float* d_out, float* delta,
                           int qHeads, int headDim, int strideColumns, int colStart,
@@ -92,6 +110,12 @@ int sentinel_oracle_layer(const float* x, const float* wq, const float* wk, cons
                           const float* d_y, float* y, float* d_x, float* d_wq, float* d_wk, float* d_wv, float* d_wo,
                           int embeddingDim, int qHeads, int kvHeads, int headDim, int seqLen, float ropeBase,
                           int ropePositions);
+
+/* the layer with the sparse mask of sentinel_oracle_attention_sparse (the host layer's windowSize / globalTokenCount) */
+int sentinel_oracle_layer_sparse(const float* x, const float* wq, const float* wk, const float* wv, const float* wo,
+                                 const float* d_y, float* y, float* d_x, float* d_wq, float* d_wk, float* d_wv, float* d_wo,
+                                 int embeddingDim, int qHeads, int kvHeads, int headDim, int seqLen, float ropeBase,
+                                 int ropePositions, int windowSize, int globalTokenCount);
 
 int sentinel_oracle_max_threads(void);
 

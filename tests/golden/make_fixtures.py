@@ -104,6 +104,52 @@ def main():
             lay[f"{tag}_{key}"] = val
     np.savez_compressed(os.path.join(HERE, "layer_kat.npz"), **lay)
     print("layer_kat", len(lay), "arrays")
+    write_sparse_kat()
+
+
+# name: (q_heads, kv_heads, head_dim, seq_len, packs, window, global_tokens)
+SPARSE_CASES = {
+    "smoke_h2_d16_T16_W4_G2": (2, 2, 16, 16, 1, 4, 2),    # runSparseComputeSmokeDemo(32, 2, 16, 32, 4, 2)
+    "gqa_4q2kv_d8_T50_W7_G0": (4, 2, 8, 50, 1, 7, 0),      # window only, grouped heads
+    "h1_d64_T140_W33_G5": (1, 1, 64, 140, 2, 33, 5),        # several 64-wide tiles, two packs
+    "h2_d32_T70_W0_G9": (2, 2, 32, 70, 1, 0, 9),            # no window: the global tokens change nothing
+    "h1_d128_T130_W1_G0": (1, 1, 128, 130, 1, 1, 0),        # window 1: every query sees only itself
+    "h1_d16_T40_W100_G3": (1, 1, 16, 40, 1, 100, 3),        # window wider than the sequence
+}
+
+
+def write_sparse_kat():
+    """Sliding-window / global-token masks from the reference's dense masked path (preferSparseCompute = false),
+    plus the forward of its sparse-compute path, which differs only by summation order."""
+    rng = np.random.default_rng(0x5E17 + 50)
+    kat = {}
+    for tag, (hq, hkv, d, t, packs, window, global_tokens) in SPARSE_CASES.items():
+        stride = packs * t
+        q = rng.standard_normal((hq * d, stride)).astype(np.float32)
+        k = rng.standard_normal((hkv * d, stride)).astype(np.float32)
+        v = rng.standard_normal((hkv * d, stride)).astype(np.float32)
+        g = rng.standard_normal((hq * d, stride)).astype(np.float32)
+        kw = dict(q_heads=hq, kv_heads=hkv, head_dim=d, seq_len=t, pack_count=packs, window=window,
+                  global_tokens=global_tokens, lib="ref")
+        # a window of 0 means "none" to the layer's constructor only through windowSize >= sequence length
+        ref_kw = dict(kw, window=window if window > 0 else t)
+        dense = oracle_lib.oracle_attention(q, k, v, g, prefer_sparse=False, **ref_kw)
+        sparse = oracle_lib.oracle_attention(q, k, v, g, prefer_sparse=True, **ref_kw)
+        kat[f"{tag}_geometry"] = np.array([hq, hkv, d, t, packs, window, global_tokens], dtype=np.int64)
+        for key, val in dict(q=q, k=k, v=v, d_out=g).items():
+            kat[f"{tag}_{key}"] = val
+        for key, val in dense.items():
+            kat[f"{tag}_dense_{key}"] = val
+        for key, val in sparse.items():
+            kat[f"{tag}_sparse_{key}"] = val
+    np.savez_compressed(os.path.join(HERE, "sparse_kat.npz"), **kat)
+    print("sparse_kat", len(kat), "arrays")
+
 
 if __name__ == "__main__":
-    main()
+    if sys.argv[1:] == ["sparse"]:  # only the sparse-mask known answers
+        if oracle_lib.reference() is None:
+            raise SystemExit("oracle/_ref is not built (needs the reference checkout): make -C oracle ref")
+        write_sparse_kat()
+    else:
+        main()

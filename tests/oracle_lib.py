@@ -42,6 +42,8 @@ def oracle():
         lib = ctypes.CDLL(build_oracle())
         lib.sentinel_oracle_attention.argtypes = [_fp] * 9 + [ctypes.c_int] * 7 + [ctypes.c_float, ctypes.c_int, ctypes.c_int]
         lib.sentinel_oracle_attention.restype = ctypes.c_int
+        lib.sentinel_oracle_attention_sparse.argtypes = lib.sentinel_oracle_attention.argtypes + [ctypes.c_int, ctypes.c_int]
+        lib.sentinel_oracle_layer_sparse.argtypes = [_fp] * 12 + [ctypes.c_int] * 5 + [ctypes.c_float] + [ctypes.c_int] * 3
         lib.sentinel_oracle_delta.argtypes = [_fp] * 3 + [ctypes.c_int] * 6
         lib.sentinel_oracle_gemm.argtypes = [_fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int]
         lib.sentinel_oracle_softmax_columns.argtypes = [_fp, _fp, ctypes.c_int, ctypes.c_int]
@@ -61,6 +63,7 @@ def reference():
             return None
         lib = ctypes.CDLL(REF_SO)
         lib.sentinel_ref_attention.argtypes = [_fp] * 9 + [ctypes.c_int] * 8
+        lib.sentinel_ref_attention_sparse.argtypes = [_fp] * 9 + [ctypes.c_int] * 10
         lib.sentinel_ref_gemm.argtypes = [_fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int, _fp, ctypes.c_int, ctypes.c_int]
         lib.sentinel_ref_softmax_columns.argtypes = [_fp, _fp, ctypes.c_int, ctypes.c_int]
         lib.sentinel_ref_rope_tables.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, _fp, _fp]
@@ -75,8 +78,12 @@ def _alloc_like(x, fill=np.nan):
 
 
 def oracle_attention(q, k, v, d_out=None, *, q_heads, kv_heads, head_dim, seq_len, pack_count=1, col_start=0,
-                     scale=None, causal=True, pack_parallel=False, lib="oracle", per_head=False):
+                     scale=None, causal=True, pack_parallel=False, lib="oracle", per_head=False, window=0, global_tokens=0,
+                     prefer_sparse=False):
     """Run forward (+ backward when d_out is given). Returns dict(out, lse[, dq, dk, dv]).
+
+    window / global_tokens: Sentinel's sparse mask on top of the causal one (0, 0 = full causal). With lib="ref",
+    prefer_sparse picks the reference's sparse-compute path instead of its dense masked path.
 
     Untouched columns (outside the pack window) come back as NaN so tests can check they were left alone.
     """
@@ -90,9 +97,16 @@ def oracle_attention(q, k, v, d_out=None, *, q_heads, kv_heads, head_dim, seq_le
     if d_out is not None:
         dq, dk, dv = _alloc_like(q), _alloc_like(k), _alloc_like(v)
     if lib == "oracle":
-        rc = oracle().sentinel_oracle_attention(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out), _ptr(dq),
-                                                 _ptr(dk), _ptr(dv), q_heads, kv_heads, head_dim, stride, col_start,
-                                                 seq_len, pack_count, float(scale), int(causal), int(pack_parallel))
+        rc = oracle().sentinel_oracle_attention_sparse(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out),
+                                                        _ptr(dq), _ptr(dk), _ptr(dv), q_heads, kv_heads, head_dim, stride,
+                                                        col_start, seq_len, pack_count, float(scale), int(causal),
+                                                        int(pack_parallel), int(window), int(global_tokens))
+    elif window > 0 or global_tokens > 0:
+        assert causal and abs(float(scale) - 1.0 / np.sqrt(head_dim)) < 1e-7
+        rc = reference().sentinel_ref_attention_sparse(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out),
+                                                        _ptr(dq), _ptr(dk), _ptr(dv), q_heads, kv_heads, head_dim, stride,
+                                                        col_start, seq_len, pack_count, int(window), int(global_tokens),
+                                                        int(prefer_sparse))
     else:
         assert causal and abs(float(scale) - 1.0 / np.sqrt(head_dim)) < 1e-7
         rc = reference().sentinel_ref_attention(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out), _ptr(dq),
@@ -167,7 +181,7 @@ def ref_rope_rotate(x, heads, head_dim, positions, base=10000.0, inverse=False):
 
 
 def layer(x, wq, wk, wv, wo, d_y=None, *, q_heads, kv_heads, head_dim, rope_base=10000.0, rope_positions=None,
-          lib="oracle"):
+          lib="oracle", window=0, global_tokens=0):
     """The attention layer (projections, RoPE, causal attention, output projection) on one sequence x [E, T].
 
     Returns dict(y[, d_x, d_wq, d_wk, d_wv, d_wo])."""
@@ -177,9 +191,15 @@ def layer(x, wq, wk, wv, wo, d_y=None, *, q_heads, kv_heads, head_dim, rope_base
     grads = [None] * 5
     if d_y is not None:
         grads = [np.empty_like(x), np.empty_like(wq), np.empty_like(wk), np.empty_like(wv), np.empty_like(wo)]
-    fn = oracle().sentinel_oracle_layer if lib == "oracle" else reference().sentinel_ref_layer
-    rc = fn(_ptr(x), _ptr(wq), _ptr(wk), _ptr(wv), _ptr(wo), _ptr(d_y), _ptr(y), *[_ptr(a) for a in grads], e, q_heads,
-            kv_heads, head_dim, t, float(rope_base), rope_positions)
+    if lib == "oracle":
+        rc = oracle().sentinel_oracle_layer_sparse(_ptr(x), _ptr(wq), _ptr(wk), _ptr(wv), _ptr(wo), _ptr(d_y), _ptr(y),
+                                                    *[_ptr(a) for a in grads], e, q_heads, kv_heads, head_dim, t,
+                                                    float(rope_base), rope_positions, int(window), int(global_tokens))
+    else:
+        assert window == 0 and global_tokens == 0
+        rc = reference().sentinel_ref_layer(_ptr(x), _ptr(wq), _ptr(wk), _ptr(wv), _ptr(wo), _ptr(d_y), _ptr(y),
+                                            *[_ptr(a) for a in grads], e, q_heads, kv_heads, head_dim, t, float(rope_base),
+                                            rope_positions)
     if rc != 0:
         raise ValueError(f"{lib} layer returned {rc}")
     res = {"y": y}
