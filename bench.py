@@ -292,6 +292,47 @@ def decode_path(torch, steps):
     return report
 
 
+def sparse_path(torch, name, steps):
+    """The step under the attention layer's sliding-window + global-token mask at the same shape: time and the
+    matrix-core rate on the visible (query, key) pairs only, 14 * d FLOPs per pair (7 products of 2 * d)."""
+    import sentinel_amd
+    b, hq, hkv, t, d, dtype, _, _ = CONFIGS[name]
+    q, k, v, g = make_inputs(torch, name)
+    out = torch.empty_like(q)
+    lse = torch.empty(b, hq, t, dtype=torch.float32, device="cuda")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    delta = torch.empty(hq, b * t, dtype=torch.float32, device="cuda")
+    report = {}
+    for window, global_tokens in ((t // 8, 0), (t // 8, 64), (t // 32, 0), (t // 2, 0)):
+        kw = dict(window_size=window, global_token_count=global_tokens)
+
+        def step():
+            sentinel_amd.flash_attention_forward(q, k, v, out=out, lse=lse, **kw)
+            sentinel_amd.flash_attention_backward(q, k, v, out, lse, g, dq=dq, dk=dk, dv=dv, delta=delta, **kw)
+
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        sentinel_amd.set_kernel_timing(True)
+        sentinel_amd.collect_kernel_timings()
+        for _ in range(steps):
+            step()
+        times = sentinel_amd.collect_kernel_timings()
+        sentinel_amd.set_kernel_timing(False)
+        pairs = sum(min(qi + 1, window) + min(global_tokens, max(qi + 1 - window, 0)) for qi in range(t))
+        flops = 14.0 * d * pairs * b * hq
+        report[f"W{window}_G{global_tokens}"] = {
+            "ms_per_step": ms, "visible_pairs_fraction_of_causal": pairs / (t * (t + 1) / 2.0),
+            "tflops_on_visible_pairs": flops / (ms * 1e-3) / 1e12,
+            "kernels_ms": {kname: tot / max(n, 1) for kname, (tot, n) in times.items()}}
+    return report
+
+
 def rocminfo_gpu_clock_ghz():
     """Max Clock Freq. of the first gfx agent as printed by rocminfo (GHz), 0.0 if it cannot be read."""
     import re
@@ -319,6 +360,8 @@ def main():
     ap.add_argument("--columns-path", action="store_true",
                     help="also time the step through Sentinel's fp32 column layout (conversion passes, fused rotary "
                          "embedding) and report it under \"columns_path\"")
+    ap.add_argument("--sparse-path", action="store_true",
+                    help="also time the step under sliding-window + global-token masks and report it under \"sparse_path\"")
     ap.add_argument("--decode-path", action="store_true",
                     help="also time single-query attention against a K/V cache (generation) and report it under \"decode_path\"")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -423,6 +466,9 @@ def main():
         del w
         torch.cuda.empty_cache()
         line["columns_path"] = columns_path(torch, args.config, max(args.steps // 5, 3), rope=True)
+
+    if args.sparse_path:
+        line["sparse_path"] = sparse_path(torch, args.config, max(args.steps // 2, 5))
 
     if args.decode_path:
         line["decode_path"] = decode_path(torch, max(args.steps, 20))

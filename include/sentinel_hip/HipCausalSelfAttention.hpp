@@ -16,8 +16,10 @@
 // CudaCausalSelfAttention::prefill / decode (Cuda/CudaCausalSelfAttention.cu:549-575): the rotated K and V columns
 // are appended to the cache and the single query of a decode step attends to it with sentinel_hip_decode_attention
 // in place of attendCachedQuery's per-head copies and GEMMs (:318-341).
-// Not built: the dense materialising fallback (sliding-window / global-token masks, flash disabled); those
-// configurations throw std::runtime_error instead of running something else.
+// Layers with a sliding window / global tokens (windowSize, globalTokenCount) run on the same kernels with the
+// sparse mask (sentinel_hip_flash_fwd_sparse / _bwd_sparse), where the CUDA class falls back to its dense path.
+// Not built: that dense materialising fallback itself (preferFlashAttention = false throws std::runtime_error
+// instead of running something else).
 // Link against libsentinel_hip_attn.so, rocBLAS and the HIP runtime.
 #ifndef SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
 #define SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
@@ -200,13 +202,17 @@ public:
     }
 
     /// CudaCausalSelfAttention::canUseFlashAttention (Cuda/CudaCausalSelfAttention.cu:46-57) without the
-    /// multiple-of-4 rules, which these kernels do not need
+    /// multiple-of-4 rules and without the full-causal-only rule, neither of which these kernels need
     bool canUseFlashAttention(int sequenceLength) const {
+        (void)sequenceLength;
         if (!preferFlashAttention) return false;
         if (headDimension <= 0 || headDimension > HipFlashAttention::maxHeadDimension) return false;
-        if (windowSize > 0 && windowSize < sequenceLength) return false;
         return true;
     }
+
+    /// the sparse mask is in force for sequences longer than the window (CausalSelfAttention::usesSparseCompute's
+    /// rule, Layers/CausalSelfAttention.cpp:102-107; shorter ones see the plain causal mask)
+    bool usesSparseMask(int sequenceLength) const { return windowSize > 0 && windowSize < sequenceLength; }
 
     /// causal multi head attention writing into out; input is embeddingDim x columns, packs of segmentLength columns
     void forward(const HipMatrix& input, HipMatrix& out, int segmentLength = 0) {
@@ -219,7 +225,7 @@ public:
         if (columns % segmentLength != 0) throw std::invalid_argument(std::string(op) + " columns must be a multiple of segmentLength");
         if (segmentLength > maximumPositionCount) throw std::invalid_argument(std::string(op) + " segmentLength exceeds RoPE table");
         if (!canUseFlashAttention(segmentLength))
-            throw std::runtime_error(std::string(op) + " needs the dense attention path (sparse window or flash disabled), which is not built");
+            throw std::runtime_error(std::string(op) + " needs the dense attention path (flash disabled), which is not built");
         activeSegmentLength = segmentLength;
         activePackCount = columns / segmentLength;
         usedFlashAttention = true;
@@ -232,14 +238,26 @@ public:
         HipGemm::multiplyInto(keyWeight, input, key);
         HipGemm::multiplyInto(valueWeight, input, value);
         const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
+        const bool sparse = usesSparseMask(segmentLength);
         if (fusedRotation()) {
-            HipFlashAttention::forwardMultiHeadRope(query, key, value, attended, flashLogSumExp, cosTable, sinTable, 0, headCount,
-                                                    headDimension, scale, true, 0, segmentLength, activePackCount, kvHeadCount);
+            if (sparse)
+                HipFlashAttention::forwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, &cosTable, &sinTable, 0,
+                                                          windowSize, globalTokenCount, headCount, headDimension, scale, 0,
+                                                          segmentLength, activePackCount, kvHeadCount);
+            else
+                HipFlashAttention::forwardMultiHeadRope(query, key, value, attended, flashLogSumExp, cosTable, sinTable, 0,
+                                                        headCount, headDimension, scale, true, 0, segmentLength,
+                                                        activePackCount, kvHeadCount);
         } else {
             HipOps::rotaryRotateInPlace(query, headCount, headDimension, pairCount, cosTable, sinTable, 0, segmentLength);
             HipOps::rotaryRotateInPlace(key, kvHeadCount, headDimension, pairCount, cosTable, sinTable, 0, segmentLength);
-            HipFlashAttention::forwardMultiHead(query, key, value, attended, flashLogSumExp, headCount, headDimension, scale, true,
-                                                0, segmentLength, activePackCount, kvHeadCount);
+            if (sparse)
+                HipFlashAttention::forwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, nullptr, nullptr, 0,
+                                                          windowSize, globalTokenCount, headCount, headDimension, scale, 0,
+                                                          segmentLength, activePackCount, kvHeadCount);
+            else
+                HipFlashAttention::forwardMultiHead(query, key, value, attended, flashLogSumExp, headCount, headDimension, scale,
+                                                    true, 0, segmentLength, activePackCount, kvHeadCount);
         }
         HipGemm::multiplyInto(outputWeight, attended, out);
     }
@@ -254,15 +272,29 @@ public:
         HipGemm::multiplyInto(outputGradient, attended, outputWeightGradient, false, true);
         HipGemm::multiplyInto(outputWeight, outputGradient, attendedGradient, true, false);
         const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
+        const bool sparse = usesSparseMask(activeSegmentLength);
         if (fusedRotation()) {
-            HipFlashAttention::backwardMultiHeadRope(query, key, value, attended, flashLogSumExp, attendedGradient, queryGradient,
-                                                     keyGradient, valueGradient, flashDelta, cosTable, sinTable, 0, headCount,
+            if (sparse)
+                HipFlashAttention::backwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, attendedGradient,
+                                                           queryGradient, keyGradient, valueGradient, flashDelta, &cosTable,
+                                                           &sinTable, 0, windowSize, globalTokenCount, headCount, headDimension,
+                                                           scale, 0, activeSegmentLength, activePackCount, kvHeadCount);
+            else
+                HipFlashAttention::backwardMultiHeadRope(query, key, value, attended, flashLogSumExp, attendedGradient,
+                                                         queryGradient, keyGradient, valueGradient, flashDelta, cosTable,
+                                                         sinTable, 0, headCount, headDimension, scale, true, 0,
+                                                         activeSegmentLength, activePackCount, kvHeadCount);
+        } else {
+            if (sparse)
+                HipFlashAttention::backwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, attendedGradient,
+                                                           queryGradient, keyGradient, valueGradient, flashDelta, nullptr,
+                                                           nullptr, 0, windowSize, globalTokenCount, headCount, headDimension,
+                                                           scale, 0, activeSegmentLength, activePackCount, kvHeadCount);
+            else
+                HipFlashAttention::backwardMultiHead(query, key, value, attended, flashLogSumExp, attendedGradient,
+                                                     queryGradient, keyGradient, valueGradient, flashDelta, headCount,
                                                      headDimension, scale, true, 0, activeSegmentLength, activePackCount,
                                                      kvHeadCount);
-        } else {
-            HipFlashAttention::backwardMultiHead(query, key, value, attended, flashLogSumExp, attendedGradient, queryGradient,
-                                                 keyGradient, valueGradient, flashDelta, headCount, headDimension, scale, true, 0,
-                                                 activeSegmentLength, activePackCount, kvHeadCount);
             HipOps::rotaryRotateInverseInPlace(queryGradient, headCount, headDimension, pairCount, cosTable, sinTable, 0,
                                                activeSegmentLength);
             HipOps::rotaryRotateInverseInPlace(keyGradient, kvHeadCount, headDimension, pairCount, cosTable, sinTable, 0,
@@ -285,13 +317,18 @@ public:
         if (static_cast<int>(input.cols) > maximumPositionCount)
             throw std::invalid_argument(std::string(op) + " sequence longer than maximumPositionCount");
         if (!canUseFlashAttention(static_cast<int>(input.cols)))
-            throw std::runtime_error(std::string(op) + " needs the dense attention path (sparse window or flash disabled), which is not built");
+            throw std::runtime_error(std::string(op) + " needs the dense attention path (flash disabled), which is not built");
         cache.ensureCapacity(static_cast<int>(keyWeight.rows), maximumPositionCount);
         projectAndRotate(input, 0);
         cache.append(key, value);
         const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
-        HipFlashAttention::forwardMultiHead(query, key, value, attended, flashLogSumExp, headCount, headDimension, scale, true, 0,
-                                            static_cast<int>(input.cols), 1, kvHeadCount);
+        if (usesSparseMask(static_cast<int>(input.cols)))
+            HipFlashAttention::forwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, nullptr, nullptr, 0, windowSize,
+                                                      globalTokenCount, headCount, headDimension, scale, 0,
+                                                      static_cast<int>(input.cols), 1, kvHeadCount);
+        else
+            HipFlashAttention::forwardMultiHead(query, key, value, attended, flashLogSumExp, headCount, headDimension, scale, true,
+                                                0, static_cast<int>(input.cols), 1, kvHeadCount);
         HipGemm::multiplyInto(outputWeight, attended, out);
     }
 

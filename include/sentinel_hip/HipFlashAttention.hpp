@@ -238,6 +238,73 @@ public:
                                           causal ? 1 : 0, ws, wsBytes, activeStream()));
     }
 
+    /// forwardMultiHead under the attention layer's sparse mask (windowSize, globalTokenCount of
+    /// CausalSelfAttention::allowsKey, Layers/CausalSelfAttention.cpp:95-100), which the CUDA layer can only run on
+    /// its dense path. cosTable / sinTable may be null: no rotation; otherwise as forwardMultiHeadRope.
+    static void forwardMultiHeadSparse(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, HipMatrix& out,
+                                       HipMatrix& logSumExp, const HipMatrix* cosTable, const HipMatrix* sinTable,
+                                       int positionOffset, int windowSize, int globalTokenCount, int headCount,
+                                       int headDimension, float scale, int columnStart = 0, int columnCount = 0,
+                                       int packCount = 1, int kvHeadCount = 0) {
+        const char* op = "HipFlashAttention::forwardMultiHeadSparse";
+        const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
+        if ((cosTable == nullptr) != (sinTable == nullptr)) throw std::invalid_argument(std::string(op) + " empty tables");
+        if (cosTable && (cosTable->empty() || sinTable->empty())) throw std::invalid_argument(std::string(op) + " empty tables");
+        if (!sentinel_hip_device_available()) throw std::runtime_error(std::string(op) + " no HIP device");
+        out.ensureSize(query.rows, query.cols);
+        logSumExp.ensureSize(static_cast<size_t>(headCount), query.cols);
+        void* ws = nullptr;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws);
+        check(sentinel_hip_flash_fwd_sparse(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
+                                            out.buffer.deviceData, logSumExp.buffer.deviceData,
+                                            cosTable ? cosTable->buffer.deviceData : nullptr,
+                                            sinTable ? sinTable->buffer.deviceData : nullptr,
+                                            cosTable ? static_cast<int>(cosTable->rows) : 0, positionOffset, windowSize,
+                                            globalTokenCount, SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS,
+                                            headCount, kvHeads, headDimension, static_cast<int>(query.cols), columnStart,
+                                            columnCount, packCount, scale, 1, ws, wsBytes, activeStream()));
+    }
+
+    /// backwardMultiHead under the same mask; with tables, queryGradient / keyGradient come back rotated back.
+    static void backwardMultiHeadSparse(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value,
+                                        const HipMatrix& out, const HipMatrix& logSumExp, const HipMatrix& outGradient,
+                                        HipMatrix& queryGradient, HipMatrix& keyGradient, HipMatrix& valueGradient,
+                                        HipMatrix& deltaWorkspace, const HipMatrix* cosTable, const HipMatrix* sinTable,
+                                        int positionOffset, int windowSize, int globalTokenCount, int headCount,
+                                        int headDimension, float scale, int columnStart = 0, int columnCount = 0,
+                                        int packCount = 1, int kvHeadCount = 0) {
+        const char* op = "HipFlashAttention::backwardMultiHeadSparse";
+        const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
+        if (out.rows != query.rows || out.cols != query.cols) throw std::invalid_argument(std::string(op) + " out shape mismatch");
+        if (outGradient.rows != query.rows || outGradient.cols != query.cols)
+            throw std::invalid_argument(std::string(op) + " outGradient shape mismatch");
+        if (logSumExp.rows != static_cast<size_t>(headCount) || logSumExp.cols != query.cols)
+            throw std::invalid_argument(std::string(op) + " logSumExp shape mismatch");
+        if ((cosTable == nullptr) != (sinTable == nullptr)) throw std::invalid_argument(std::string(op) + " empty tables");
+        if (cosTable && (cosTable->empty() || sinTable->empty())) throw std::invalid_argument(std::string(op) + " empty tables");
+        if (!sentinel_hip_device_available()) throw std::runtime_error(std::string(op) + " no HIP device");
+        if (packCount <= 0) packCount = 1;
+        const int resolvedCount = columnCount > 0 ? columnCount : static_cast<int>(query.cols) - columnStart;
+        if (columnStart < 0 || resolvedCount <= 0 || columnStart + resolvedCount > static_cast<int>(query.cols))
+            throw std::invalid_argument("HipFlashAttention invalid column window");
+        queryGradient.ensureSize(query.rows, query.cols);
+        keyGradient.ensureSize(key.rows, key.cols);
+        valueGradient.ensureSize(value.rows, value.cols);
+        deltaWorkspace.ensureSize(static_cast<size_t>(headCount), static_cast<size_t>(packCount) * static_cast<size_t>(resolvedCount));
+        void* ws = nullptr;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws);
+        check(sentinel_hip_flash_bwd_sparse(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
+                                            out.buffer.deviceData, logSumExp.buffer.deviceData, outGradient.buffer.deviceData,
+                                            queryGradient.buffer.deviceData, keyGradient.buffer.deviceData,
+                                            valueGradient.buffer.deviceData, deltaWorkspace.buffer.deviceData,
+                                            cosTable ? cosTable->buffer.deviceData : nullptr,
+                                            sinTable ? sinTable->buffer.deviceData : nullptr,
+                                            cosTable ? static_cast<int>(cosTable->rows) : 0, positionOffset, windowSize,
+                                            globalTokenCount, SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS,
+                                            headCount, kvHeads, headDimension, static_cast<int>(query.cols), columnStart,
+                                            columnCount, packCount, scale, 1, ws, wsBytes, activeStream()));
+    }
+
 private:
     // validateMultiHeadShape (CudaFlashAttention.cu:1458-1471), K/V rows rule widened to grouped heads
     static int validateMultiHeadShape(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, int headCount,

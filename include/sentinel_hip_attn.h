@@ -140,6 +140,31 @@ SENTINEL_HIP_API int sentinel_hip_flash_bwd_rope(const void* q, const void* k, c
                                 size_t workspace_bytes, void* stream);
 
 /*
+ * The same with Sentinel's sparse attention mask on top of the causal one: a key is visible to a query iff
+ *   key <= query and (key < global_token_count or window_size <= 0 or key >= query - window_size + 1)
+ * (CausalSelfAttention::allowsKey, sentinel/NeuralNet/Layers/CausalSelfAttention.cpp:95-100; on the device
+ * CudaOps::applySparseAttentionMaskInPlace and zeroForbiddenScoreGradientsInPlace, Cuda/CudaOps.cu:1262-1275). The
+ * CUDA layer turns flash attention off for such layers (canUseFlashAttention, Cuda/CudaCausalSelfAttention.cu:46-57)
+ * and materialises T x T scores per head (:255-314); here the kernels skip the key tiles no query of a tile can
+ * see, so the work is O(T * window) instead of O(T^2). window_size <= 0 or >= seq_len is the plain causal mask (the
+ * global tokens then change nothing). causal must be 1 with a window. cos_table / sin_table may both be NULL (no
+ * rotation); otherwise as sentinel_hip_flash_fwd_rope. Workspace as for the plain calls.
+ */
+SENTINEL_HIP_API int sentinel_hip_flash_fwd_sparse(const void* q, const void* k, const void* v, void* out, float* lse,
+                                  const float* cos_table, const float* sin_table, int table_positions,
+                                  int position_offset, int window_size, int global_token_count, int io_dtype,
+                                  int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+                                  int stride_columns, int column_start, int seq_len, int pack_count, float scale,
+                                  int causal, void* workspace, size_t workspace_bytes, void* stream);
+SENTINEL_HIP_API int sentinel_hip_flash_bwd_sparse(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                                  const void* d_out, void* dq, void* dk, void* dv, float* delta,
+                                  const float* cos_table, const float* sin_table, int table_positions,
+                                  int position_offset, int window_size, int global_token_count, int io_dtype,
+                                  int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+                                  int stride_columns, int column_start, int seq_len, int pack_count, float scale,
+                                  int causal, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Generation step: attention of ONE query position (the newest token, rows q_heads*head_dim of `query`, already
  * rotated) against the first `length` positions of an append-only K/V cache in Sentinel's layout: fp32
  * [(kv_head*head_dim + dim), position] with cache_stride positions per row (CudaKvCache::key / ::value,
@@ -148,8 +173,10 @@ SENTINEL_HIP_API int sentinel_hip_flash_bwd_rope(const void* q, const void* k, c
  * Replaces the per-head loop of CudaCausalSelfAttention::attendCachedQuery
  * (Cuda/CudaCausalSelfAttention.cu:318-341; extractHead x3, GEMM, scale, mask, softmax, GEMM, writeHead per head)
  * with two launches that read the cache once; grouped-query heads share the reads. window_size /
- * global_token_count are the layer's sparse-mask parameters: only the full causal case (window_size <= 0 or
- * >= length) is built, anything else returns SENTINEL_HIP_UNSUPPORTED. Workspace: sentinel_hip_decode_workspace_bytes.
+ * global_token_count are the layer's sparse-mask parameters (applySparseAttentionMaskInPlace with
+ * queryPositionStart = length - 1, :333): the query sees positions below global_token_count and the last
+ * window_size positions, and only those parts of the cache are read; window_size <= 0 or >= length sees all.
+ * Workspace: sentinel_hip_decode_workspace_bytes.
  */
 SENTINEL_HIP_API size_t sentinel_hip_decode_workspace_bytes(int q_heads, int head_dim, int length);
 SENTINEL_HIP_API int sentinel_hip_decode_attention(const float* query, const float* key_cache, const float* value_cache, float* out,

@@ -95,7 +95,7 @@ int resolve(const char* op, int io_dtype, int compute_dtype, int layout, int q_h
     if ((long long)pack_count * seq_len > 0x7fffffffLL / 4)
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s too many columns", op);
 
-    r->g = AttnGeom{q_heads, kv_heads, head_dim, seq_len, pack_count, scale, causal ? 1 : 0};
+    r->g = AttnGeom{q_heads, kv_heads, head_dim, seq_len, pack_count, scale, causal ? 1 : 0, 0, 0};
     r->io = io_dtype;
     r->compute = compute;
     r->layout = layout;
@@ -188,15 +188,34 @@ int check_rope(const char* op, const float* cos_table, const float* sin_table, i
     return SENTINEL_HIP_OK;
 }
 
+// The layer's sparse mask (windowSize, globalTokenCount).  A window that covers the sequence is no window, and
+// without a window the global tokens change nothing: both collapse to the plain causal mask.
+struct SparseMask {
+    int window;
+    int global_tokens;
+};
+const SparseMask kNoSparseMask = {0, 0};
+
+int apply_sparse_mask(const char* op, SparseMask mask, AttnGeom* g) {
+    if (mask.global_tokens < 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s globalTokenCount must be >= 0", op);
+    if (mask.window <= 0 || mask.window >= g->seq_len) return SENTINEL_HIP_OK;
+    if (!g->causal) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s the sliding window refines the causal mask: causal must be set", op);
+    g->window = mask.window;
+    g->global_tokens = mask.global_tokens < g->seq_len ? mask.global_tokens : g->seq_len;
+    return SENTINEL_HIP_OK;
+}
+
 int flash_fwd(const char* op, const void* q, const void* k, const void* v, void* out, float* lse, int io_dtype,
               int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim, int stride_columns, int column_start,
               int seq_len, int pack_count, float scale, int causal, void* workspace, size_t workspace_bytes,
-              void* stream_ptr, RopeTables rope) {
+              void* stream_ptr, RopeTables rope, SparseMask mask = kNoSparseMask) {
     if (!q || !k || !v || !out || !lse) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
     Resolved r;
     const int rc = resolve(op, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns, column_start,
                            seq_len, pack_count, scale, causal, &r);
     if (rc != SENTINEL_HIP_OK) return rc;
+    const int mask_rc = apply_sparse_mask(op, mask, &r.g);
+    if (mask_rc != SENTINEL_HIP_OK) return mask_rc;
     if (rope.cos && !r.adapter)
         return fail(SENTINEL_HIP_UNSUPPORTED,
                     "%s the rotation is fused into the layout conversion of fp32 column tensors with 16-bit arithmetic; "
@@ -256,13 +275,16 @@ int flash_fwd(const char* op, const void* q, const void* k, const void* v, void*
 int flash_bwd(const char* op, const void* q, const void* k, const void* v, const void* out, const float* lse,
               const void* d_out, void* dq, void* dk, void* dv, float* delta, int io_dtype, int compute_dtype, int layout,
               int q_heads, int kv_heads, int head_dim, int stride_columns, int column_start, int seq_len, int pack_count,
-              float scale, int causal, void* workspace, size_t workspace_bytes, void* stream_ptr, RopeTables rope) {
+              float scale, int causal, void* workspace, size_t workspace_bytes, void* stream_ptr, RopeTables rope,
+              SparseMask mask = kNoSparseMask) {
     if (!q || !k || !v || !out || !lse || !d_out || !dq || !dk || !dv || !delta)
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
     Resolved r;
     const int rc = resolve(op, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns, column_start,
                            seq_len, pack_count, scale, causal, &r);
     if (rc != SENTINEL_HIP_OK) return rc;
+    const int mask_rc = apply_sparse_mask(op, mask, &r.g);
+    if (mask_rc != SENTINEL_HIP_OK) return mask_rc;
     if (rope.cos && !r.adapter)
         return fail(SENTINEL_HIP_UNSUPPORTED,
                     "%s the rotation is fused into the layout conversion of fp32 column tensors with 16-bit arithmetic; "
@@ -398,6 +420,47 @@ extern "C" int sentinel_hip_flash_bwd_rope(const void* q, const void* k, const v
                      stream_ptr, rope);
 }
 
+extern "C" int sentinel_hip_flash_fwd_sparse(const void* q, const void* k, const void* v, void* out, float* lse,
+                                             const float* cos_table, const float* sin_table, int table_positions,
+                                             int position_offset, int window_size, int global_token_count, int io_dtype,
+                                             int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+                                             int stride_columns, int column_start, int seq_len, int pack_count, float scale,
+                                             int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
+    const char* op = "sentinel_hip_flash_fwd_sparse";
+    RopeTables rope = {nullptr, nullptr, 0};
+    if (cos_table || sin_table) {
+        const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
+        if (rc != SENTINEL_HIP_OK) return rc;
+        if (misaligned(cos_table) || misaligned(sin_table))
+            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
+        rope = RopeTables{cos_table, sin_table, position_offset};
+    }
+    return flash_fwd(op, q, k, v, out, lse, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns,
+                     column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes, stream_ptr, rope,
+                     SparseMask{window_size, global_token_count});
+}
+
+extern "C" int sentinel_hip_flash_bwd_sparse(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                                             const void* d_out, void* dq, void* dk, void* dv, float* delta,
+                                             const float* cos_table, const float* sin_table, int table_positions,
+                                             int position_offset, int window_size, int global_token_count, int io_dtype,
+                                             int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
+                                             int stride_columns, int column_start, int seq_len, int pack_count, float scale,
+                                             int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
+    const char* op = "sentinel_hip_flash_bwd_sparse";
+    RopeTables rope = {nullptr, nullptr, 0};
+    if (cos_table || sin_table) {
+        const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
+        if (rc != SENTINEL_HIP_OK) return rc;
+        if (misaligned(cos_table) || misaligned(sin_table))
+            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
+        rope = RopeTables{cos_table, sin_table, position_offset};
+    }
+    return flash_bwd(op, q, k, v, out, lse, d_out, dq, dk, dv, delta, io_dtype, compute_dtype, layout, q_heads, kv_heads,
+                     head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes,
+                     stream_ptr, rope, SparseMask{window_size, global_token_count});
+}
+
 extern "C" int sentinel_hip_rope_rotate(float* tensor, int heads, int head_dim, int stride_columns, int column_start,
                                         int columns, int position_offset, int segment_length, const float* cos_table,
                                         const float* sin_table, int table_positions, int inverse, void* stream_ptr) {
@@ -438,9 +501,7 @@ extern "C" int sentinel_hip_decode_attention(const float* query, const float* ke
     if (length <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s cache is empty", op);
     if (length > cache_stride) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s cache length exceeds its capacity", op);
     if (!(scale > 0.0f) || !std::isfinite(scale)) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s scale must be positive and finite", op);
-    (void)global_token_count;
-    if (window_size > 0 && window_size < length)
-        return fail(SENTINEL_HIP_UNSUPPORTED, "%s sliding-window masks are not built (window %d < cache length %d)", op, window_size, length);
+    if (global_token_count < 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s globalTokenCount must be >= 0", op);
     const int group = q_heads / kv_heads;
     if (group != 1 && group != 2 && group != 4 && group != 8)
         return fail(SENTINEL_HIP_UNSUPPORTED, "%s query heads per K/V head must be 1, 2, 4 or 8 (got %d)", op, group);
@@ -450,8 +511,8 @@ extern "C" int sentinel_hip_decode_attention(const float* query, const float* ke
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s needs %zu bytes of 16-byte aligned workspace", op, need);
     if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
     const hipError_t err = launch_decode_attention(query, key_cache, value_cache, out, q_heads, kv_heads, head_dim,
-                                                   cache_stride, length, scale, static_cast<float*>(workspace),
-                                                   static_cast<hipStream_t>(stream_ptr));
+                                                   cache_stride, length, scale, window_size, global_token_count,
+                                                   static_cast<float*>(workspace), static_cast<hipStream_t>(stream_ptr));
     if (err != hipSuccess) return fail_hip("decode attention launch", err);
     return SENTINEL_HIP_OK;
 }

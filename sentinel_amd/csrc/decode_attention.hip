@@ -13,6 +13,8 @@
 // (max, sum, acc[d]) in the workspace; a second small kernel merges the partials.
 #include "flash_common.h"
 
+#include <algorithm>
+
 namespace sentinel_hip {
 namespace {
 
@@ -138,11 +140,17 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_partial_kernel(const fl
                                                                        const float* __restrict__ key_cache,
                                                                        const float* __restrict__ value_cache,
                                                                        float* __restrict__ partial, int kv_heads, int d,
-                                                                       long long stride, int length, float scale) {
+                                                                       long long stride, int length, float scale,
+                                                                       int global_tokens, int window_lo, int global_chunks,
+                                                                       int window_chunk) {
     __shared__ float exchange[kWavesPerBlock][G * PPL][64];
     const int lane = threadIdx.x % 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
-    const int chunk = blockIdx.x;
+    // Sparse mask of the layer (the query is position length - 1): visible are the global tokens [0, global_tokens)
+    // and the window [window_lo, length).  Only chunks that hold a visible position are launched: the first
+    // global_chunks ones and those from window_chunk on; partials are numbered by workgroup.
+    const int slot = blockIdx.x;
+    const int chunk = slot < global_chunks ? slot : slot - global_chunks + window_chunk;
     const int kvh = blockIdx.y;
     const int q_heads = kv_heads * G;
     const int first = chunk * (64 * PPL) + (VEC4 ? 4 * lane : lane);
@@ -190,10 +198,10 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_partial_kernel(const fl
             const float dot = (exchange[0][g * PPL + i][lane] + exchange[1][g * PPL + i][lane]) +
                               (exchange[2][g * PPL + i][lane] + exchange[3][g * PPL + i][lane]);
             const int j = first + (VEC4 ? i : 64 * i);
-            s[i][g] = j < length ? dot * scale : -__builtin_inff();
+            s[i][g] = (j < length && (j < global_tokens || j >= window_lo)) ? dot * scale : -__builtin_inff();
             m = fmaxf(m, s[i][g]);
         }
-        m = wave_max(m);  // finite: the chunk holds at least one position < length
+        m = wave_max(m);  // finite: the chunk holds at least one visible position
         float sum = 0.0f;
 #pragma unroll
         for (int i = 0; i < PPL; ++i) {
@@ -202,7 +210,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_partial_kernel(const fl
         }
         sum = wave_sum(sum);
         if (wave == 0 && lane == 0) {
-            float* out = partial + ((long long)chunk * q_heads + kvh * G + g) * (d + 2);
+            float* out = partial + ((long long)slot * q_heads + kvh * G + g) * (d + 2);
             out[0] = m;
             out[1] = sum;
         }
@@ -231,7 +239,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_partial_kernel(const fl
         // lane L now holds the total with index L % (kLoadRows * G) = (row in batch) * G + head
         const float total = reduce_scatter<kLoadRows * G>(x, lane);
         const int c = c0 + lane / G;
-        if (lane < kLoadRows * G && c < r1) partial[((long long)chunk * q_heads + kvh * G + lane % G) * (d + 2) + 2 + c] = total;
+        if (lane < kLoadRows * G && c < r1) partial[((long long)slot * q_heads + kvh * G + lane % G) * (d + 2) + 2 + c] = total;
     }
 }
 
@@ -285,9 +293,16 @@ size_t decode_workspace_bytes(int q_heads, int head_dim, int length) {
 
 hipError_t launch_decode_attention(const float* query, const float* key_cache, const float* value_cache, float* out,
                                    int q_heads, int kv_heads, int head_dim, int stride, int length, float scale,
-                                   float* workspace, hipStream_t stream) {
+                                   int window, int global_tokens, float* workspace, hipStream_t stream) {
     const int chunk = decode_chunk(length);
-    const int chunks = (length + chunk - 1) / chunk;
+    const int all_chunks = (length + chunk - 1) / chunk;
+    // window <= 0 or >= length: every position is visible
+    const bool sparse = window > 0 && window < length;
+    const int window_lo = sparse ? length - window : 0;
+    if (!sparse) global_tokens = 0;
+    const int global_chunks = sparse ? (std::min(global_tokens, window_lo) + chunk - 1) / chunk : 0;
+    const int window_chunk = std::max(global_chunks, window_lo / chunk);
+    const int chunks = global_chunks + (all_chunks - window_chunk);
     const int group = q_heads / kv_heads;
     if (head_dim % 8 != 0) return hipErrorInvalidValue;
     const dim3 grid(chunks, kv_heads);
@@ -299,13 +314,16 @@ hipError_t launch_decode_attention(const float* query, const float* key_cache, c
     do {                                                                                                                     \
         if (chunk == kSmallChunk)                                                                                            \
             hipLaunchKernelGGL((decode_partial_kernel<G, false, 1>), grid, dim3(kDecodeThreads), 0, stream, query,           \
-                               key_cache, value_cache, workspace, kv_heads, head_dim, (long long)stride, length, scale);     \
+                               key_cache, value_cache, workspace, kv_heads, head_dim, (long long)stride, length, scale,      \
+                               global_tokens, window_lo, global_chunks, window_chunk);                                       \
         else if (v4)                                                                                                         \
             hipLaunchKernelGGL((decode_partial_kernel<G, true, 4>), grid, dim3(kDecodeThreads), 0, stream, query,            \
-                               key_cache, value_cache, workspace, kv_heads, head_dim, (long long)stride, length, scale);     \
+                               key_cache, value_cache, workspace, kv_heads, head_dim, (long long)stride, length, scale,      \
+                               global_tokens, window_lo, global_chunks, window_chunk);                                       \
         else                                                                                                                 \
             hipLaunchKernelGGL((decode_partial_kernel<G, false, 4>), grid, dim3(kDecodeThreads), 0, stream, query,           \
-                               key_cache, value_cache, workspace, kv_heads, head_dim, (long long)stride, length, scale);     \
+                               key_cache, value_cache, workspace, kv_heads, head_dim, (long long)stride, length, scale,      \
+                               global_tokens, window_lo, global_chunks, window_chunk);                                       \
     } while (0)
         if (group == 1) SENTINEL_DECODE(1);
         else if (group == 2) SENTINEL_DECODE(2);

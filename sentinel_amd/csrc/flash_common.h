@@ -18,7 +18,17 @@ struct AttnGeom {
     int packs;
     float scale;
     int causal;
+    // Sentinel's sparse mask on top of the causal one (CausalSelfAttention::allowsKey,
+    // sentinel/NeuralNet/Layers/CausalSelfAttention.cpp:95-100): with window > 0 a key at or past global_tokens is
+    // visible only to the queries key .. key + window - 1.  window == 0: full causal (global_tokens is then 0 too).
+    int window;
+    int global_tokens;
 };
+
+// true when the sparse mask forbids the pair (the causal rule key <= query is checked separately)
+__host__ __device__ inline bool outside_window(const AttnGeom& g, int query, int key) {
+    return g.window > 0 && key >= g.global_tokens && query - key >= g.window;
+}
 
 // element(pack, head, t, c) = base[pack * pack_stride + head * head_stride + t * t_stride + c * c_stride]
 // Sentinel's column layout: pack_stride = seq_len, head_stride = head_dim * stride_columns, t_stride = 1,
@@ -70,9 +80,10 @@ hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int he
                                   int seq_len, int packs, RopeTables inverse_rope, hipStream_t stream);
 // single-query attention against the K/V cache (fp32 column layout, `stride` positions per row, `length` used)
 size_t decode_workspace_bytes(int q_heads, int head_dim, int length);
+// window / global_tokens: the layer's sparse mask for the query at position length - 1 (window <= 0: none)
 hipError_t launch_decode_attention(const float* query, const float* key_cache, const float* value_cache, float* out,
                                    int q_heads, int kv_heads, int head_dim, int stride, int length, float scale,
-                                   float* workspace, hipStream_t stream);
+                                   int window, int global_tokens, float* workspace, hipStream_t stream);
 // in-place rotation of fp32 column-layout rows (tensor already advanced to the first column)
 hipError_t launch_rope_rotate_f32(float* tensor, int heads, int head_dim, int stride_columns, int columns,
                                   int position_offset, int segment_length, const float* cos, const float* sin, bool inverse,

@@ -76,7 +76,11 @@ __global__ __launch_bounds__(kLanes) void fwd_f32_kernel(const float* __restrict
     float l = 0.0f;
     const int kv_end = g.causal ? min(T, tile * kLanes + kLanes) : T;
 
+    // first key any query of this tile still sees through its window (stages before it matter only for global tokens)
+    const int window_lo = g.window > 0 ? tile * kLanes - g.window + 1 : 0;
+
     for (int k0 = 0; k0 < kv_end; k0 += kKeyStage) {
+        if (k0 >= g.global_tokens && k0 + kKeyStage <= window_lo) continue;  // workgroup-uniform: nothing visible in this stage
         __syncthreads();
         stage_rows<DP, kKeyStage>(ks, kbase, km, k0, T, d, lane);
         stage_rows<DP, kKeyStage>(vs, vbase, km, k0, T, d, lane);
@@ -92,7 +96,7 @@ __global__ __launch_bounds__(kLanes) void fwd_f32_kernel(const float* __restrict
 #pragma unroll
                 for (int c = 0; c < DP; ++c) dot += qr[c] * kr[c];
                 const int kj = k0 + j0 + jj;
-                s[jj] = (kj >= T || (g.causal && kj > qi)) ? -INFINITY : dot;
+                s[jj] = (kj >= T || (g.causal && kj > qi) || outside_window(g, qi, kj)) ? -INFINITY : dot;
             }
             float mx = m;
 #pragma unroll
@@ -178,8 +182,10 @@ __global__ __launch_bounds__(kLanes) void bwd_dq_f32_kernel(const float* __restr
     const float lse2 = lse[b * lm.pack_stride + h * lm.head_stride + qload] * kLog2e;
     const float dl = delta[(long long)h * g.packs * T + (long long)b * T + qload];
     const int kv_end = g.causal ? min(T, tile * kLanes + kLanes) : T;
+    const int window_lo = g.window > 0 ? tile * kLanes - g.window + 1 : 0;
 
     for (int k0 = 0; k0 < kv_end; k0 += kKeyStage) {
+        if (k0 >= g.global_tokens && k0 + kKeyStage <= window_lo) continue;  // workgroup-uniform: nothing visible in this stage
         __syncthreads();
         stage_rows<DP, kKeyStage>(ks, kbase, km, k0, T, d, lane);
         stage_rows<DP, kKeyStage>(vs, vbase, km, k0, T, d, lane);
@@ -196,7 +202,7 @@ __global__ __launch_bounds__(kLanes) void bwd_dq_f32_kernel(const float* __restr
                 s += qr[c] * kr[c];
                 dp += gr[c] * vr[c];
             }
-            const float p = (g.causal && kj > qi) ? 0.0f : exp2f(s * c2 - lse2);
+            const float p = ((g.causal && kj > qi) || outside_window(g, qi, kj)) ? 0.0f : exp2f(s * c2 - lse2);
             const float ds = p * (dp - dl) * g.scale;
 #pragma unroll
             for (int c = 0; c < DP; ++c) acc[c] += ds * kr[c];
@@ -255,6 +261,8 @@ __global__ __launch_bounds__(kLanes) void bwd_dkdv_f32_kernel(const float* __res
     }
     const float c2 = g.scale * kLog2e;
     const int q_begin = g.causal ? ktile * kLanes : 0;
+    // a tile without global tokens is seen by the queries up to its last key + window - 1 only
+    const int q_end = (g.window > 0 && ktile * kLanes >= g.global_tokens) ? min(T, ktile * kLanes + kLanes + g.window - 1) : T;
 
     for (int gi = 0; gi < group; ++gi) {
         const int h = kvh * group + gi;
@@ -262,7 +270,7 @@ __global__ __launch_bounds__(kLanes) void bwd_dkdv_f32_kernel(const float* __res
         const float* gbase = d_out + b * qm.pack_stride + h * qm.head_stride;
         const float* lrow = lse + b * lm.pack_stride + h * lm.head_stride;
         const float* drow = delta + (long long)h * g.packs * T + (long long)b * T;
-        for (int q0 = q_begin; q0 < T; q0 += kQueryStage) {
+        for (int q0 = q_begin; q0 < q_end; q0 += kQueryStage) {
             __syncthreads();
             stage_rows<DP, kQueryStage>(qs, qbase, qm, q0, T, d, lane);
             stage_rows<DP, kQueryStage>(gs, gbase, qm, q0, T, d, lane);
@@ -284,7 +292,7 @@ __global__ __launch_bounds__(kLanes) void bwd_dkdv_f32_kernel(const float* __res
                     s += qrow[c] * kt[c * kLanes + lane];
                     dp += grow[c] * vt[c * kLanes + lane];
                 }
-                const float p = (kj >= T || (g.causal && kj > qi)) ? 0.0f : exp2f(s * c2 - lse2s[i]);
+                const float p = (kj >= T || (g.causal && kj > qi) || outside_window(g, qi, kj)) ? 0.0f : exp2f(s * c2 - lse2s[i]);
                 const float ds = p * (dp - dls[i]) * g.scale;
 #pragma unroll
                 for (int c = 0; c < DP; ++c) {

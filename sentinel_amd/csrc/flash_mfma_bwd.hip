@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kBwdThreads) void delta_mfma_kernel(const unsigned 
 constexpr int kDqQueryTile = 128;
 constexpr int kDqKeyTile = 64;
 
-template <typename E, int D, bool CAUSAL>
+template <typename E, int D, bool CAUSAL, bool WINDOW>
 __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned short* __restrict__ q,
                                                                   const unsigned short* __restrict__ k,
                                                                   const unsigned short* __restrict__ v,
@@ -124,12 +124,23 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 
     const int q_hi = min(T, (qt + 1) * kDqQueryTile);
     const int kv_tiles = CAUSAL ? (q_hi + KT - 1) / KT : (T + KT - 1) / KT;
+    // WINDOW (Sentinel's sliding window + global tokens on top of the causal mask): the key tiles this query tile
+    // sees are those holding global tokens, [0, g_tiles), and those from the window of its first query up to the
+    // diagonal, [w_first, kv_tiles); trip `it` works on tile_of(it)
+    static_assert(CAUSAL || !WINDOW, "the sparse mask refines the causal one");
+    int g_tiles = 0, w_first = 0;
+    if (WINDOW) {
+        g_tiles = min(kv_tiles, (g.global_tokens + KT - 1) / KT);
+        w_first = max(g_tiles, max(0, qt * kDqQueryTile - g.window + 1) / KT);
+    }
+    const int n_trips = WINDOW ? g_tiles + (kv_tiles - w_first) : kv_tiles;
+    auto tile_of = [&](int it) { return WINDOW ? (it < g_tiles ? it : it - g_tiles + w_first) : it; };
 
     const __amdgpu_buffer_rsrc_t k_rsrc = make_head_rsrc(kb, (long long)T * D * 2);
     const __amdgpu_buffer_rsrc_t v_rsrc = make_head_rsrc(vb, (long long)T * D * 2);
     const int ld_off = Tile::global_offset(tid);
-    Tile::issue(k_rsrc, k_lds0, ld_off, 0, wave);
-    Tile::issue(v_rsrc, v_lds0, ld_off, 0, wave);
+    Tile::issue(k_rsrc, k_lds0, ld_off, tile_of(0) * KT * D * 2, wave);
+    Tile::issue(v_rsrc, v_lds0, ld_off, tile_of(0) * KT * D * 2, wave);
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
         pin_loaded(qf[ks]);
@@ -148,6 +159,10 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
         for (int i = 0; i < 16; ++i) acc[cb][i] = 0.0f;
 
     const int mask_base = (CAUSAL ? min(qrow, T - 1) : T - 1) - 2 * gh;  // last live key of this lane's query, minus the lane half's row offset
+    // sparse mask: a key is dead when it is no global token and lies window or more before the query, i.e. when
+    // global_base <= key - 2 gh <= window_base
+    const int global_base = g.global_tokens - 2 * gh;
+    const int window_base = qrow - g.window - 2 * gh;
     const int k_off = Tile::row_read_base(row_perm(n), gh);
     const int t_even = Tile::transposed_read_base(lane, 0);
     const int t_odd = Tile::transposed_read_base(lane, 1);
@@ -157,13 +172,16 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     auto tile_trip = [&](auto masked_tag, int j, const unsigned short* kt, const unsigned short* vt, unsigned short* kt_next,
                          unsigned short* vt_next) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        const bool more = j + 1 < kv_tiles;
+        const bool more = j + 1 < n_trips;
         if (more) {
-            Tile::issue(k_rsrc, kt_next, ld_off, (j + 1) * KT * D * 2, wave);
-            Tile::issue(v_rsrc, vt_next, ld_off, (j + 1) * KT * D * 2, wave);
+            Tile::issue(k_rsrc, kt_next, ld_off, tile_of(j + 1) * KT * D * 2, wave);
+            Tile::issue(v_rsrc, vt_next, ld_off, tile_of(j + 1) * KT * D * 2, wave);
         }
-        const int key0 = j * KT;
-        const bool skip = MASKED && CAUSAL && key0 > q0w + 31;
+        const int key0 = tile_of(j) * KT;
+        // wavefront-uniform: the whole tile lies above this wavefront's diagonal, or holds no global token and
+        // lies below the window of this wavefront's first query
+        const bool skip = MASKED && CAUSAL &&
+                          (key0 > q0w + 31 || (WINDOW && key0 >= g.global_tokens && key0 + KT - 1 < q0w - g.window + 1));
         if (!skip) {
             // two 32-key halves one after the other keeps the live score registers to one half
 #pragma unroll
@@ -203,6 +221,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                     p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -lse2));
                     // dead iff key0 + 32 kbk + (row of register i in lane half 0) + 2 gh > last live key
                     if (MASKED && perm_row_of_reg(i, 0) > mask_base - key0 - kbk * 32) p[i] = 0.0f;
+                    if (MASKED && WINDOW && perm_row_of_reg(i, 0) >= global_base - key0 - kbk * 32 &&
+                        perm_row_of_reg(i, 0) <= window_base - key0 - kbk * 32)
+                        p[i] = 0.0f;
                 }
                 u32x4 dsf[2];
 #pragma unroll
@@ -243,14 +264,15 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 
     // Tiles that end at or before the first query of the workgroup need no mask for any wavefront; keep the count
     // even so that the masked tail starts on LDS stage 0 again.
-    const int bare_tiles = (CAUSAL ? min(kv_tiles, qt * (kDqQueryTile / KT)) : T / KT) & ~1;
+    // Under the sparse mask a query tile sees few tiles and most of them cross a mask edge: all trips are masked ones.
+    const int bare_tiles = WINDOW ? 0 : (CAUSAL ? min(kv_tiles, qt * (kDqQueryTile / KT)) : T / KT) & ~1;
     for (int j = 0; j < bare_tiles; j += 2) {
         tile_trip(std::false_type{}, j, k_lds0, v_lds0, k_lds1, v_lds1);
         tile_trip(std::false_type{}, j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
     }
-    for (int j = bare_tiles; j < kv_tiles; j += 2) {
+    for (int j = bare_tiles; j < n_trips; j += 2) {
         tile_trip(std::true_type{}, j, k_lds0, v_lds0, k_lds1, v_lds1);
-        if (j + 1 < kv_tiles) tile_trip(std::true_type{}, j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
+        if (j + 1 < n_trips) tile_trip(std::true_type{}, j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
     }
 
     if (qrow < T) {
@@ -320,7 +342,47 @@ struct DkvLds {
     float dl[QT];
 };
 
-template <typename E, int D, bool CAUSAL>
+// Stage ranges of one query head for a wavefront whose 32 keys start at k0w, under the causal mask and, with
+// WINDOW, Sentinel's sparse mask: stages [first, causal_end) cross the causal diagonal, stages [upper_begin, end)
+// hold queries that lie window or more behind one of the wavefront's keys outside the global range; both kinds
+// take the masked code, what lies between runs bare.
+struct DkvMaskedRanges {
+    int causal_end;
+    int upper_begin;
+};
+template <bool CAUSAL, bool WINDOW>
+__device__ __forceinline__ DkvMaskedRanges dkv_masked_ranges(const AttnGeom& g, int k0w, int first, int end, int q_first,
+                                                             int n_qt) {
+    constexpr int QT = 64;
+    DkvMaskedRanges r;
+    r.causal_end = first;
+    r.upper_begin = end;
+    if (k0w + 31 >= g.seq_len) {  // keys past the end of the sequence: every stage masks them
+        r.causal_end = end;
+        return r;
+    }
+    if (CAUSAL) r.causal_end = min(end, first + max(0, (k0w + 31 + QT - 1) / QT - q_first));
+    if (WINDOW) {
+        const int kmin = max(k0w, g.global_tokens);  // first key of the wavefront the window applies to
+        if (kmin <= k0w + 31) r.upper_begin = max(r.causal_end, first + min(n_qt, max(0, (kmin + g.window) / QT - q_first)));
+    }
+    return r;
+}
+
+// Query tiles a key tile of 128 keys starting at k0 meets: from its causal diagonal to the end of the sequence, or,
+// with the sparse mask and no global token in the tile, to the last query whose window still reaches the tile.
+template <bool CAUSAL, bool WINDOW>
+__device__ __forceinline__ int dkv_query_tiles(const AttnGeom& g, int k0, int q_first) {
+    constexpr int QT = 64;
+    const int q_tiles_all = (g.seq_len + QT - 1) / QT;
+    if (WINDOW && k0 >= g.global_tokens) {
+        const long long last_query = (long long)k0 + 127 + g.window - 1;
+        if (last_query < g.seq_len) return (int)(last_query / QT) + 1 - q_first;
+    }
+    return q_tiles_all - q_first;
+}
+
+template <typename E, int D, bool CAUSAL, bool WINDOW>
 __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
@@ -368,9 +430,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     }
     const float c2 = g.scale * kLog2e;
 
-    const int q_tiles_all = (T + QT - 1) / QT;
+    static_assert(QT == 64 && kDkvKeyTile == 128, "dkv_query_tiles / dkv_masked_ranges assume these tiles");
     const int q_first = CAUSAL ? (ktile * kDkvKeyTile) / QT : 0;
-    const int n_qt = q_tiles_all - q_first;
+    const int n_qt = dkv_query_tiles<CAUSAL, WINDOW>(g, ktile * kDkvKeyTile, q_first);
     const int n_iter = group * n_qt;
 
     f32x16 dk_acc[CB];
@@ -459,7 +521,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
                     float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -l2[i]));
                     if (MASKED) {
                         const int query = q0b + perm_row_of_reg(i, gh);
-                        if ((CAUSAL && key > query) || key_dead) p = 0.0f;
+                        if ((CAUSAL && key > query) || key_dead || (WINDOW && outside_window(g, query, key))) p = 0.0f;
                     }
                     p2[w] = p;
                     ds2[w] = p * (dp[i] - dl[i]);
@@ -525,13 +587,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
         int it = 0;
         for (int gi = 0; gi < group; ++gi) {
             const int head_end = (gi + 1) * n_qt;
-            int masked_end = it;
-            if (k0w + 31 >= T)
-                masked_end = head_end;
-            else if (CAUSAL)
-                masked_end = min(head_end, it + max(0, (k0w + 31 + QT - 1) / QT - q_first));
-            for (; it < masked_end; ++it) stage_trip(std::true_type{}, it);
-            for (; it < head_end; ++it) stage_trip(std::false_type{}, it);
+            const DkvMaskedRanges r = dkv_masked_ranges<CAUSAL, WINDOW>(g, k0w, it, head_end, q_first, n_qt);
+            for (; it < r.causal_end; ++it) stage_trip(std::true_type{}, it);
+            for (; it < r.upper_begin; ++it) stage_trip(std::false_type{}, it);
+            if (WINDOW)
+                for (; it < head_end; ++it) stage_trip(std::true_type{}, it);
         }
     }
 
@@ -553,7 +613,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     }
 }
 
-template <typename E, int D, bool CAUSAL>
+template <typename E, int D, bool CAUSAL, bool WINDOW>
 __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
@@ -602,9 +662,9 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     }
     const float c2 = g.scale * kLog2e;
 
-    const int q_tiles_all = (T + QT - 1) / QT;
+    static_assert(QT == 64 && kDkvKeyTile == 128, "dkv_query_tiles / dkv_masked_ranges assume these tiles");
     const int q_first = CAUSAL ? (ktile * kDkvKeyTile) / QT : 0;
-    const int n_qt = q_tiles_all - q_first;
+    const int n_qt = dkv_query_tiles<CAUSAL, WINDOW>(g, ktile * kDkvKeyTile, q_first);
     const int n_iter = group * n_qt;
 
     f32x16 acc[CB];  // dV^T (score role) or dK^T (grad role)
@@ -726,6 +786,9 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         // key - query of register i, block blk is mask_rel - (32 blk + row of register i in lane half 0): one
         // per-lane value compared against compile-time constants; a key past the end masks everything
         const int mask_rel = key_dead ? 0x7fffffff : (CAUSAL ? key - q0 - gh * 2 : -0x7fffffff);
+        // sparse mask: a key outside the global range is dead for queries window or more behind it, i.e. from
+        // 32 blk + row = mask_rel + window on
+        const int window_rel = (WINDOW && !key_dead && key >= g.global_tokens) ? mask_rel + g.window : 0x7fffffff;
         u32x4 qrow[KSTEPS];
         u32x4 gcol[2][CB];
         f32x16 s;
@@ -750,6 +813,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
                         const int i = half * 8 + 2 * e + w;
                         float p = __builtin_amdgcn_exp2f(s[i] * c2);
                         if (MASKED && mask_rel > blk * 32 + perm_row_of_reg(i, 0)) p = 0.0f;
+                        if (MASKED && WINDOW && window_rel <= blk * 32 + perm_row_of_reg(i, 0)) p = 0.0f;
                         p2[w] = p;
                     }
                     pf[half][e] = E::pack2(p2[0], p2[1]);
@@ -828,13 +892,11 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         int it = 0;
         for (int gi = 0; gi < group; ++gi) {
             const int head_end = (gi + 1) * n_qt;
-            int masked_end = it;
-            if (k0w + 31 >= T)
-                masked_end = head_end;
-            else if (CAUSAL)
-                masked_end = min(head_end, it + max(0, (k0w + 31 + QT - 1) / QT - q_first));
-            for (; it < masked_end; ++it) score_trip(std::true_type{}, it);
-            for (; it < head_end; ++it) score_trip(std::false_type{}, it);
+            const DkvMaskedRanges r = dkv_masked_ranges<CAUSAL, WINDOW>(g, k0w, it, head_end, q_first, n_qt);
+            for (; it < r.causal_end; ++it) score_trip(std::true_type{}, it);
+            for (; it < r.upper_begin; ++it) score_trip(std::false_type{}, it);
+            if (WINDOW)
+                for (; it < head_end; ++it) score_trip(std::true_type{}, it);
         }
         __syncthreads();
     } else {
@@ -887,12 +949,15 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
         const int grid = (total + 7) / 8 * 8;
         const size_t smem = 2 * sizeof(DkvLds<D>);
         KernelTimer timer("dkdv_mfma", stream);
-        if (g.causal)
-            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, true>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp,
-                               lse, delta, dkp, dvp, lm, g, k_tiles, total);
+        if (g.window > 0)
+            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, true, true>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp,
+                               gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
+        else if (g.causal)
+            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, true, false>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp,
+                               gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
         else
-            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, false>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp,
-                               lse, delta, dkp, dvp, lm, g, k_tiles, total);
+            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, false, false>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp,
+                               vp, gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     } else {
@@ -900,22 +965,26 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
         const int total = g.packs * g.kv_heads * k_tiles;
         const int grid = (total + 7) / 8 * 8;
         const size_t smem = sizeof(DkvSplitLds<D>);
-        static bool raised[2] = {false, false};  // one-time opt-in to more than 64 KiB of LDS per kernel
-        const int which = g.causal ? 1 : 0;
+        static bool raised[3] = {false, false, false};  // one-time opt-in to more than 64 KiB of LDS per kernel
+        const int which = g.window > 0 ? 2 : g.causal ? 1 : 0;
         if (!raised[which]) {
-            const void* fn = g.causal ? reinterpret_cast<const void*>(dkdv_split_kernel<E, D, true>)
-                                      : reinterpret_cast<const void*>(dkdv_split_kernel<E, D, false>);
+            const void* fn = which == 2   ? reinterpret_cast<const void*>(dkdv_split_kernel<E, D, true, true>)
+                             : which == 1 ? reinterpret_cast<const void*>(dkdv_split_kernel<E, D, true, false>)
+                                          : reinterpret_cast<const void*>(dkdv_split_kernel<E, D, false, false>);
             err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
             if (err != hipSuccess) return err;
             raised[which] = true;
         }
         KernelTimer timer("dkdv_mfma", stream);
-        if (g.causal)
-            hipLaunchKernelGGL((dkdv_split_kernel<E, D, true>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp,
-                               gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
+        if (which == 2)
+            hipLaunchKernelGGL((dkdv_split_kernel<E, D, true, true>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp,
+                               kp, vp, gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
+        else if (which == 1)
+            hipLaunchKernelGGL((dkdv_split_kernel<E, D, true, false>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp,
+                               kp, vp, gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
         else
-            hipLaunchKernelGGL((dkdv_split_kernel<E, D, false>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp,
-                               gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
+            hipLaunchKernelGGL((dkdv_split_kernel<E, D, false, false>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp,
+                               kp, vp, gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
@@ -925,12 +994,15 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
         const int total = g.packs * g.q_heads * q_tiles;
         const int grid = (total + 7) / 8 * 8;
         KernelTimer timer("dq_mfma", stream);
-        if (g.causal)
-            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp, lse,
-                               delta, dqp, lm, g, q_tiles, total);
+        if (g.window > 0)
+            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true, true>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp,
+                               lse, delta, dqp, lm, g, q_tiles, total);
+        else if (g.causal)
+            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp,
+                               lse, delta, dqp, lm, g, q_tiles, total);
         else
-            hipLaunchKernelGGL((dq_mfma_kernel<E, D, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp, lse,
-                               delta, dqp, lm, g, q_tiles, total);
+            hipLaunchKernelGGL((dq_mfma_kernel<E, D, false, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp,
+                               lse, delta, dqp, lm, g, q_tiles, total);
         err = hipGetLastError();
     }
     return err;

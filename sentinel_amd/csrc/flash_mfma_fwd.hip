@@ -13,7 +13,8 @@
 //     out of the row-major V tile with transposing LDS reads;
 //   * the running maximum is only raised (and O rescaled) when a row's maximum grows by more than 2^8,
 //     which is exact and keeps P within the 16-bit range;
-//   * key tiles above the diagonal are skipped; only tiles that cross it are masked;
+//   * key tiles above the diagonal are skipped; only tiles that cross it are masked; with Sentinel's sparse mask
+//     (sliding window + global tokens, WINDOW) the key tiles below every window of the query tile are skipped too;
 //   * grouped-query attention reads the shared K/V head in place.
 #include "flash_common.h"
 #include "mfma_tile.h"
@@ -30,7 +31,7 @@ constexpr int kOperandLead = 4;
 
 constexpr int kFwdKeyTile = 64;
 
-template <typename E, int D, bool CAUSAL>
+template <typename E, int D, bool CAUSAL, bool WINDOW>
 __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned short* __restrict__ q,
                                                                    const unsigned short* __restrict__ k,
                                                                    const unsigned short* __restrict__ v,
@@ -82,6 +83,16 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
 
     const int q_hi = min(T, (qt + 1) * kFwdQueryTile);        // one past the last query of the tile
     const int kv_tiles = CAUSAL ? (q_hi + KT - 1) / KT : (T + KT - 1) / KT;
+    // WINDOW: the key tiles this query tile sees are the ones holding global tokens, [0, g_tiles), and those from
+    // the window of its first query up to the diagonal, [w_first, kv_tiles); trip `it` works on tile_of(it)
+    static_assert(CAUSAL || !WINDOW, "the sparse mask refines the causal one");
+    int g_tiles = 0, w_first = 0;
+    if (WINDOW) {
+        g_tiles = min(kv_tiles, (g.global_tokens + KT - 1) / KT);
+        w_first = max(g_tiles, max(0, qt * kFwdQueryTile - g.window + 1) / KT);
+    }
+    const int n_trips = WINDOW ? g_tiles + (kv_tiles - w_first) : kv_tiles;
+    auto tile_of = [&](int it) { return WINDOW ? (it < g_tiles ? it : it - g_tiles + w_first) : it; };
 
     const __amdgpu_buffer_rsrc_t k_rsrc = make_head_rsrc(kb, (long long)T * D * 2);
     const __amdgpu_buffer_rsrc_t v_rsrc = make_head_rsrc(vb, (long long)T * D * 2);
@@ -90,8 +101,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     const int v_st = VTile::lds_offset(tid);
     KTile kt;
     VTile vt;
-    kt.load(k_rsrc, ld_off, 0);
-    vt.load(v_rsrc, ld_off, 0);
+    kt.load(k_rsrc, ld_off, tile_of(0) * KT * D * 2);
+    vt.load(v_rsrc, ld_off, tile_of(0) * KT * D * 2);
     kt.store(k_lds[0], k_st);
     vt.store(v_lds[0], v_st);
 #pragma unroll
@@ -103,7 +114,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[cb][i] = 0.0f;
-    float m_run = -__builtin_inff();
+    // Under the sparse mask a row can meet a tile in which all its keys are masked before it meets a visible key:
+    // a finite floor keeps exp2(-inf - m) = 0 there instead of exp2(-inf + inf)
+    float m_run = WINDOW ? -1e30f : -__builtin_inff();
     float l_run = 0.0f;  // this lane's half of the row sum
     const float c2 = g.scale * kLog2e;
 
@@ -111,17 +124,19 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     const int v_off = transposed_read_offset(lane, VS);  // V^T operand read out of the row-major tile
     const float raise_after = 8.0f;                // log2 units a row maximum may grow before O is rescaled
 
-    for (int j = 0; j < kv_tiles; ++j) {
+    for (int j = 0; j < n_trips; ++j) {
         const int buf = j & 1;
-        const bool more = j + 1 < kv_tiles;
+        const bool more = j + 1 < n_trips;
         if (more) {
-            kt.load(k_rsrc, ld_off, (j + 1) * KT * D * 2);
-            vt.load(v_rsrc, ld_off, (j + 1) * KT * D * 2);
+            kt.load(k_rsrc, ld_off, tile_of(j + 1) * KT * D * 2);
+            vt.load(v_rsrc, ld_off, tile_of(j + 1) * KT * D * 2);
         }
 
-        const int key0 = j * KT;
-        // wavefront-uniform: the whole tile lies above this wavefront's diagonal
-        const bool skip = CAUSAL && key0 > q0w + 31;
+        const int key0 = tile_of(j) * KT;
+        // wavefront-uniform: the whole tile lies above this wavefront's diagonal, or holds no global token and
+        // lies below the window of this wavefront's first query
+        const bool skip = (CAUSAL && key0 > q0w + 31) ||
+                          (WINDOW && key0 >= g.global_tokens && key0 + KT - 1 < q0w - g.window + 1);
         if (!skip) {
             // S^T chains with their K operands read kOperandLead instructions ahead; the V^T operands of the first
             // half of the PV product are fetched behind them and land during the softmax arithmetic
@@ -157,14 +172,16 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             }
             __builtin_amdgcn_sched_barrier(0);
 
-            const bool need_mask = (CAUSAL && key0 + KT - 1 > q0w) || (!CAUSAL && key0 + KT > T);
+            // also when the tile's first key outside the global range lies below the window of the wavefront's last query
+            const bool need_mask = (CAUSAL && key0 + KT - 1 > q0w) || (!CAUSAL && key0 + KT > T) ||
+                                   (WINDOW && key0 + KT > g.global_tokens && max(key0, g.global_tokens) < q0w + 32 - g.window);
             if (need_mask) {
 #pragma unroll
                 for (int kbk = 0; kbk < 2; ++kbk)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int key = key0 + kbk * 32 + perm_row_of_reg(i, gh);
-                        const bool dead = CAUSAL ? key > qrow : key >= T;
+                        const bool dead = CAUSAL ? (key > qrow || (WINDOW && outside_window(g, qrow, key))) : key >= T;
                         if (dead) s[kbk][i] = -__builtin_inff();
                     }
             }
@@ -261,12 +278,15 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
     auto vp = static_cast<const unsigned short*>(v);
     auto op = static_cast<unsigned short*>(out);
     KernelTimer timer("fwd_mfma", stream);
-    if (g.causal)
-        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, true>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm,
-                           g, q_tiles, total);
+    if (g.window > 0)
+        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, true, true>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op,
+                           lse, lm, g, q_tiles, total);
+    else if (g.causal)
+        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, true, false>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op,
+                           lse, lm, g, q_tiles, total);
     else
-        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, false>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm,
-                           g, q_tiles, total);
+        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, false, false>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op,
+                           lse, lm, g, q_tiles, total);
     return hipGetLastError();
 }
 

@@ -55,6 +55,10 @@ def load_library():
     lib.sentinel_hip_flash_fwd_rope.restype = i
     lib.sentinel_hip_flash_bwd_rope.argtypes = [vp] * 12 + [i] * 12 + [f, i, vp, sz, vp]
     lib.sentinel_hip_flash_bwd_rope.restype = i
+    lib.sentinel_hip_flash_fwd_sparse.argtypes = [vp] * 7 + [i] * 14 + [f, i, vp, sz, vp]
+    lib.sentinel_hip_flash_fwd_sparse.restype = i
+    lib.sentinel_hip_flash_bwd_sparse.argtypes = [vp] * 12 + [i] * 14 + [f, i, vp, sz, vp]
+    lib.sentinel_hip_flash_bwd_sparse.restype = i
     lib.sentinel_hip_rope_rotate.argtypes = [vp] + [i] * 7 + [vp, vp, i, i, vp]
     lib.sentinel_hip_rope_rotate.restype = i
     lib.sentinel_hip_decode_workspace_bytes.argtypes = [i] * 3
@@ -182,8 +186,11 @@ class HipFlashAttention:
     @staticmethod
     def forward_multi_head(query, key, value, out, log_sum_exp, head_count, head_dimension, scale, causal=True,
                            column_start=0, column_count=0, pack_count=1, *, kv_head_count=None, compute=None,
-                           workspace=None, stream=None, rope=None):
+                           workspace=None, stream=None, rope=None, window_size=0, global_token_count=0):
         """CudaFlashAttention::forwardMultiHead. Returns (out, log_sum_exp) (re-allocated if their shape was wrong).
+
+        window_size / global_token_count: the attention layer's sparse mask (CausalSelfAttention::allowsKey), which
+        the CUDA layer can only run on its dense path.
 
         rope = (cos_table, sin_table[, position_offset]): query and key are given unrotated and rotated on the way in
         (the two rotaryRotateInPlace calls of CudaCausalSelfAttention.cu:206-207 fused into this call)."""
@@ -199,7 +206,12 @@ class HipFlashAttention:
                                   max(pack_count, 1), False, query.device, workspace)
         tail = (F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start, column_count,
                 pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes, _stream_handle(stream))
-        if rope is None:
+        if window_size > 0 or global_token_count != 0:
+            cos, sin, offset = _rope_args(rope, head_dimension) if rope is not None else (None, None, 0)
+            _check(lib.sentinel_hip_flash_fwd_sparse(_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp),
+                                                     _ptr(cos), _ptr(sin), int(cos.shape[0]) if cos is not None else 0,
+                                                     offset, int(window_size), int(global_token_count), *tail))
+        elif rope is None:
             _check(lib.sentinel_hip_flash_fwd(_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp), *tail))
         else:
             cos, sin, offset = _rope_args(rope, head_dimension)
@@ -217,7 +229,7 @@ class HipFlashAttention:
     def backward_multi_head(query, key, value, out, log_sum_exp, out_gradient, query_gradient, key_gradient,
                             value_gradient, delta_workspace, head_count, head_dimension, scale, causal=True,
                             column_start=0, column_count=0, pack_count=1, *, kv_head_count=None, compute=None,
-                            workspace=None, stream=None, rope=None):
+                            workspace=None, stream=None, rope=None, window_size=0, global_token_count=0):
         """CudaFlashAttention::backwardMultiHead. Returns (dQ, dK, dV, delta).
 
         rope as in forward_multi_head: query / key unrotated, dQ / dK come back rotated back
@@ -245,7 +257,11 @@ class HipFlashAttention:
                 _ptr(key_gradient), _ptr(value_gradient), _ptr(delta_workspace))
         tail = (F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start, column_count,
                 pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes, _stream_handle(stream))
-        if rope is None:
+        if window_size > 0 or global_token_count != 0:
+            cos, sin, offset = _rope_args(rope, head_dimension) if rope is not None else (None, None, 0)
+            _check(lib.sentinel_hip_flash_bwd_sparse(*head, _ptr(cos), _ptr(sin), int(cos.shape[0]) if cos is not None else 0,
+                                                     offset, int(window_size), int(global_token_count), *tail))
+        elif rope is None:
             _check(lib.sentinel_hip_flash_bwd(*head, *tail))
         else:
             cos, sin, offset = _rope_args(rope, head_dimension)
@@ -328,7 +344,8 @@ def _bhtd_geometry(q, k, v):
     return b, hq, k.shape[1], t, d
 
 
-def flash_attention_forward(q, k, v, scale=None, causal=True, out=None, lse=None, stream=None):
+def flash_attention_forward(q, k, v, scale=None, causal=True, out=None, lse=None, stream=None, window_size=0,
+                            global_token_count=0):
     """Native forward on [B,H,T,d] tensors (k, v may have fewer heads). Returns (out, lse[B,H,T] fp32)."""
     lib = load_library()
     b, hq, hkv, t, d = _bhtd_geometry(q, k, v)
@@ -336,13 +353,19 @@ def flash_attention_forward(q, k, v, scale=None, causal=True, out=None, lse=None
     out = torch.empty_like(q) if out is None else out
     lse = torch.empty((b, hq, t), dtype=torch.float32, device=q.device) if lse is None else lse
     code = _DTYPE_CODE[q.dtype]
+    if window_size > 0 or global_token_count != 0:
+        _check(lib.sentinel_hip_flash_fwd_sparse(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), None, None, 0, 0,
+                                                 int(window_size), int(global_token_count), code, COMPUTE_AUTO, LAYOUT_BHTD,
+                                                 hq, hkv, d, 0, 0, t, b, scale, int(bool(causal)), None, 0,
+                                                 _stream_handle(stream)))
+        return out, lse
     _check(lib.sentinel_hip_flash_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), code, COMPUTE_AUTO, LAYOUT_BHTD, hq,
                                       hkv, d, 0, 0, t, b, scale, int(bool(causal)), None, 0, _stream_handle(stream)))
     return out, lse
 
 
 def flash_attention_backward(q, k, v, out, lse, d_out, scale=None, causal=True, dq=None, dk=None, dv=None, delta=None,
-                             stream=None):
+                             stream=None, window_size=0, global_token_count=0):
     """Native backward on [B,H,T,d] tensors. Returns (dq, dk, dv)."""
     lib = load_library()
     b, hq, hkv, t, d = _bhtd_geometry(q, k, v)
@@ -352,7 +375,10 @@ def flash_attention_backward(q, k, v, out, lse, d_out, scale=None, causal=True, 
     dv = torch.empty_like(v) if dv is None else dv
     delta = torch.empty((hq, b * t), dtype=torch.float32, device=q.device) if delta is None else delta
     code = _DTYPE_CODE[q.dtype]
-    _check(lib.sentinel_hip_flash_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out), _ptr(dq), _ptr(dk),
-                                      _ptr(dv), _ptr(delta), code, COMPUTE_AUTO, LAYOUT_BHTD, hq, hkv, d, 0, 0, t, b, scale,
-                                      int(bool(causal)), None, 0, _stream_handle(stream)))
+    head = (_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(delta))
+    tail = (code, COMPUTE_AUTO, LAYOUT_BHTD, hq, hkv, d, 0, 0, t, b, scale, int(bool(causal)), None, 0, _stream_handle(stream))
+    if window_size > 0 or global_token_count != 0:
+        _check(lib.sentinel_hip_flash_bwd_sparse(*head, None, None, 0, 0, int(window_size), int(global_token_count), *tail))
+    else:
+        _check(lib.sentinel_hip_flash_bwd(*head, *tail))
     return dq, dk, dv

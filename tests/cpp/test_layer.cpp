@@ -40,7 +40,8 @@ static void expectThrow(const char* what, Fn fn) {
     throw std::runtime_error(std::string("expected an exception: ") + what);
 }
 
-static void runCase(const char* name, int e, int heads, int kvHeads, int d, int T, int packs, int compute, float tol) {
+static void runCase(const char* name, int e, int heads, int kvHeads, int d, int T, int packs, int compute, float tol,
+                    int windowSize = 0, int globalTokenCount = 0) {
     const int qRows = heads * d, kvRows = kvHeads * d, cols = packs * T;
     unsigned state = 2024u + static_cast<unsigned>(e + T);
     const float bound = 1.0f / std::sqrt(static_cast<float>(e));
@@ -54,6 +55,8 @@ static void runCase(const char* name, int e, int heads, int kvHeads, int d, int 
     host.kvHeadCount = kvHeads;
     host.headDimension = d;
     host.maximumPositionCount = T + 5;
+    host.windowSize = windowSize;
+    host.globalTokenCount = globalTokenCount;
     auto hx = lcg(static_cast<size_t>(e) * cols, state, 1.0f);
     auto hg = lcg(static_cast<size_t>(e) * cols, state, 1.0f);
 
@@ -68,9 +71,10 @@ static void runCase(const char* name, int e, int heads, int kvHeads, int d, int 
                 x[static_cast<size_t>(r) * T + c] = hx[static_cast<size_t>(r) * cols + p * T + c];
                 g[static_cast<size_t>(r) * T + c] = hg[static_cast<size_t>(r) * cols + p * T + c];
             }
-        if (sentinel_oracle_layer(x.data(), host.queryWeight.data(), host.keyWeight.data(), host.valueWeight.data(),
-                                  host.outputWeight.data(), g.data(), y.data(), dx.data(), dq.data(), dk.data(), dv.data(),
-                                  dwo.data(), e, heads, kvHeads, d, T, host.ropeBase, host.maximumPositionCount) != 0)
+        if (sentinel_oracle_layer_sparse(x.data(), host.queryWeight.data(), host.keyWeight.data(), host.valueWeight.data(),
+                                         host.outputWeight.data(), g.data(), y.data(), dx.data(), dq.data(), dk.data(),
+                                         dv.data(), dwo.data(), e, heads, kvHeads, d, T, host.ropeBase,
+                                         host.maximumPositionCount, windowSize, globalTokenCount) != 0)
             throw std::runtime_error("oracle layer failed");
         for (int r = 0; r < e; ++r)
             for (int c = 0; c < T; ++c) {
@@ -101,7 +105,8 @@ static void runCase(const char* name, int e, int heads, int kvHeads, int d, int 
 // Generation: prefill `prompt` columns, then decode the rest one token at a time. Step t must reproduce column t of
 // the oracle's full forward over columns 0..t (causal attention: earlier columns do not depend on later ones, so
 // one oracle call over all columns gives every step's answer).
-static void runGeneration(const char* name, int e, int heads, int kvHeads, int d, int prompt, int total, int compute, float tol) {
+static void runGeneration(const char* name, int e, int heads, int kvHeads, int d, int prompt, int total, int compute, float tol,
+                          int windowSize = 0, int globalTokenCount = 0) {
     const int qRows = heads * d, kvRows = kvHeads * d;
     unsigned state = 4711u + static_cast<unsigned>(e + total);
     const float bound = 1.0f / std::sqrt(static_cast<float>(e));
@@ -115,11 +120,14 @@ static void runGeneration(const char* name, int e, int heads, int kvHeads, int d
     host.kvHeadCount = kvHeads;
     host.headDimension = d;
     host.maximumPositionCount = total;
+    host.windowSize = windowSize;
+    host.globalTokenCount = globalTokenCount;
     auto hx = lcg(static_cast<size_t>(e) * total, state, 1.0f);
     std::vector<float> want(hx.size());
-    if (sentinel_oracle_layer(hx.data(), host.queryWeight.data(), host.keyWeight.data(), host.valueWeight.data(),
-                              host.outputWeight.data(), nullptr, want.data(), nullptr, nullptr, nullptr, nullptr, nullptr, e, heads,
-                              kvHeads, d, total, host.ropeBase, host.maximumPositionCount) != 0)
+    if (sentinel_oracle_layer_sparse(hx.data(), host.queryWeight.data(), host.keyWeight.data(), host.valueWeight.data(),
+                                     host.outputWeight.data(), nullptr, want.data(), nullptr, nullptr, nullptr, nullptr, nullptr, e,
+                                     heads, kvHeads, d, total, host.ropeBase, host.maximumPositionCount, windowSize,
+                                     globalTokenCount) != 0)
         throw std::runtime_error("oracle layer failed");
 
     HipFlashAttention::computeType() = compute;
@@ -165,12 +173,20 @@ int main() {
         // MFMA arithmetic for the attention core (projections stay fp32), rotation fused into the conversion passes
         runCase("bf16 E256 H4 d64 T128 packs2", 256, 4, 4, 64, 128, 2, SENTINEL_HIP_COMPUTE_BF16, 2e-2f);
         runCase("fp16 GQA E256 4q/1kv d128 T200", 256, 4, 1, 128, 200, 1, SENTINEL_HIP_COMPUTE_F16, 2e-2f);
+        // the sparse mask: the shape of runSparseComputeSmokeDemo (E=32, H=2, T=16, W=4, G=2) and larger ones
+        HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
+        runCase("sparse fp32 E32 H2 d16 T16 W4 G2", 32, 2, 2, 16, 16, 1, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 4, 2);
+        runCase("sparse fp32 GQA 8q/2kv d8 T90 W17 G3 packs2", 64, 8, 2, 8, 90, 2, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 17, 3);
+        runCase("sparse bf16 E256 H4 d64 T300 W70 G10", 256, 4, 4, 64, 300, 1, SENTINEL_HIP_COMPUTE_BF16, 2e-2f, 70, 10);
+        runCase("sparse fp16 GQA 4q/1kv d128 T200 W33 packs2", 256, 4, 1, 128, 200, 2, SENTINEL_HIP_COMPUTE_F16, 2e-2f, 33, 0);
         HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
         // the shapes of runKvCacheSmokeDemo (E=64, H=4, T=32 of 64 positions), grouped heads, a cache of several chunks
         runGeneration("generate fp32 E64 H4 d16 32+32", 64, 4, 4, 16, 32, 64, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
         runGeneration("generate fp32 GQA 8q/2kv d8 5+20", 64, 8, 2, 8, 5, 25, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
         runGeneration("generate fp32 E128 H2 d64 1+300", 128, 2, 2, 64, 1, 301, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
         runGeneration("generate bf16 prefill GQA 4q/1kv d128", 256, 4, 1, 128, 130, 140, SENTINEL_HIP_COMPUTE_BF16, 2e-2f);
+        runGeneration("generate sparse fp32 H4 d16 20+60 W9 G2", 64, 4, 4, 16, 20, 80, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 9, 2);
+        runGeneration("generate sparse fp32 GQA d64 3+400 W100 G70", 128, 4, 2, 64, 3, 403, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 100, 70);
         HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
 
         // configurations this layer does not run are refused, not approximated
@@ -184,13 +200,12 @@ int main() {
         host.keyWeight = host.queryWeight;
         host.valueWeight = host.queryWeight;
         host.outputWeight = host.queryWeight;
-        host.windowSize = 4;
-        HipCausalSelfAttention sparse = HipCausalSelfAttention::createFrom(host);
+        HipCausalSelfAttention noFlash = HipCausalSelfAttention::createFrom(host);
+        noFlash.preferFlashAttention = false;
         HipMatrix x, y;
         x.ensureSize(32, 16);
         x.fill(0.1f);
-        expectThrow("sliding window needs the dense path", [&] { sparse.forward(x, y); });
-        host.windowSize = 0;
+        expectThrow("flash disabled needs the dense path", [&] { noFlash.forward(x, y); });
         HipCausalSelfAttention dense = HipCausalSelfAttention::createFrom(host);
         expectThrow("columns not a multiple of the segment", [&] { dense.forward(x, y, 5); });
         HipMatrix longer;

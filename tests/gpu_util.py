@@ -33,9 +33,10 @@ def bht_to_columns(y, heads, stride, col0):
     return brute.bht_to_ref(y.detach().float().cpu().numpy(), stride=stride, col0=col0)
 
 
-def oracle(q, k, v, g, hq, hkv, d, t, packs, col0=0, causal=True, scale=None):
+def oracle(q, k, v, g, hq, hkv, d, t, packs, col0=0, causal=True, scale=None, window=0, global_tokens=0):
     return oracle_lib.oracle_attention(q, k, v, g, q_heads=hq, kv_heads=hkv, head_dim=d, seq_len=t, pack_count=packs,
-                                       col_start=col0, causal=causal, scale=scale, pack_parallel=True)
+                                       col_start=col0, causal=causal, scale=scale, pack_parallel=True, window=window,
+                                       global_tokens=global_tokens)
 
 
 def assert_close_fp32(got, want, name, tol=1e-4):
