@@ -6,8 +6,9 @@
 //     a loop-invariant vector offset (the hardware range check zero-fills rows past T); nothing is
 //     converted or gathered per tile;
 //   * a workgroup of 4 wavefronts owns 128 queries (32 per wavefront) and walks 64-key tiles;
-//     Q stays in registers for the whole kernel, K and V tiles are double-buffered in LDS (row-major)
-//     and the next tile's global loads are in flight while the current one is multiplied;
+//     Q stays in registers for the whole kernel, K and V tiles are double-buffered in LDS (row-major,
+//     XOR-swizzled) and the next tile streams straight into LDS (buffer_load ... lds) while the current one
+//     is multiplied;
 //   * S^T = K Q^T, so a lane owns one query: the online-softmax max / sum are in-register plus one
 //     v_permlane32_swap, and P^T feeds the P V product from registers (no LDS round trip); V^T is read
 //     out of the row-major V tile with transposing LDS reads;
@@ -39,15 +40,12 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
                                                                    float* __restrict__ lse, RowMap lm, AttnGeom g,
                                                                    int q_tiles, int total_tiles) {
     constexpr int KT = kFwdKeyTile;
-    typedef RowTile<KT, D, kFwdThreads, 8> KTile;
-    typedef RowTile<KT, D, kFwdThreads, 8> VTile;
-    constexpr int KS = KTile::kStride;
-    constexpr int VS = VTile::kStride;
+    typedef DirectTile<KT, D, kFwdThreads> Tile;
     constexpr int KSTEPS = D / 16;  // k-steps of the S^T product
     constexpr int CB = D / 32;      // 32-row blocks of O^T
 
-    __shared__ __attribute__((aligned(16))) unsigned short k_lds[2][KT * KS];
-    __shared__ __attribute__((aligned(16))) unsigned short v_lds[2][KT * VS];
+    __shared__ __attribute__((aligned(16))) unsigned short k_lds[2][Tile::kElems];
+    __shared__ __attribute__((aligned(16))) unsigned short v_lds[2][Tile::kElems];
 
     // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of tiles so
     // that the q-tiles of one head (which stream the same K/V) share one L2.
@@ -96,17 +94,12 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
 
     const __amdgpu_buffer_rsrc_t k_rsrc = make_head_rsrc(kb, (long long)T * D * 2);
     const __amdgpu_buffer_rsrc_t v_rsrc = make_head_rsrc(vb, (long long)T * D * 2);
-    const int ld_off = KTile::global_offset(tid);
-    const int k_st = KTile::lds_offset(tid);
-    const int v_st = VTile::lds_offset(tid);
-    KTile kt;
-    VTile vt;
-    kt.load(k_rsrc, ld_off, tile_of(0) * KT * D * 2);
-    vt.load(v_rsrc, ld_off, tile_of(0) * KT * D * 2);
-    kt.store(k_lds[0], k_st);
-    vt.store(v_lds[0], v_st);
+    const int ld_off = Tile::global_offset(tid);
+    Tile::issue(k_rsrc, k_lds[0], ld_off, tile_of(0) * KT * D * 2, wave);
+    Tile::issue(v_rsrc, v_lds[0], ld_off, tile_of(0) * KT * D * 2, wave);
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) pin_loaded(qf[ks]);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the first tiles have landed in LDS
     __syncthreads();
 
     f32x16 acc[CB];
@@ -120,16 +113,17 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     float l_run = 0.0f;  // this lane's half of the row sum
     const float c2 = g.scale * kLog2e;
 
-    const int k_off = row_perm(n) * KS + gh * 8;  // K operand read: row carried by D row n
-    const int v_off = transposed_read_offset(lane, VS);  // V^T operand read out of the row-major tile
+    const int k_off = Tile::row_read_base(row_perm(n), gh);  // K operand read: row carried by D row n
+    const int t_even = Tile::transposed_read_base(lane, 0);  // V^T operand reads out of the row-major V tile
+    const int t_odd = Tile::transposed_read_base(lane, 1);
     const float raise_after = 8.0f;                // log2 units a row maximum may grow before O is rescaled
 
     for (int j = 0; j < n_trips; ++j) {
         const int buf = j & 1;
         const bool more = j + 1 < n_trips;
         if (more) {
-            kt.load(k_rsrc, ld_off, tile_of(j + 1) * KT * D * 2);
-            vt.load(v_rsrc, ld_off, tile_of(j + 1) * KT * D * 2);
+            Tile::issue(k_rsrc, k_lds[buf ^ 1], ld_off, tile_of(j + 1) * KT * D * 2, wave);
+            Tile::issue(v_rsrc, v_lds[buf ^ 1], ld_off, tile_of(j + 1) * KT * D * 2, wave);
         }
 
         const int key0 = tile_of(j) * KT;
@@ -146,7 +140,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
 #pragma unroll
             for (int kbk = 0; kbk < 2; ++kbk)
 #pragma unroll
-                for (int ks = 0; ks < KSTEPS; ++ks) kfrag[kbk][ks] = lds_read128(&k_lds[buf][kbk * 32 * KS + k_off + ks * 16]);
+                for (int ks = 0; ks < KSTEPS; ++ks) kfrag[kbk][ks] = lds_read128(&k_lds[buf][kbk * 32 * D + (k_off ^ (ks << 4))]);
 #pragma unroll
             for (int kbk = 0; kbk < 2; ++kbk) {
 #pragma unroll
@@ -158,7 +152,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             for (int c4 = 0; c4 < 2; ++c4)
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
-                    vfrag[c4][cb] = lds_read_transposed(&v_lds[buf][v_off + c4 * 16 * VS + cb * 32], VS);
+                    vfrag[c4][cb] = lds_read_transposed_pair(&v_lds[buf][c4 * 16 * D + (t_even ^ (cb << 5))],
+                                                             &v_lds[buf][c4 * 16 * D + (t_odd ^ (cb << 5))]);
             __builtin_amdgcn_sched_group_barrier(kSchedDsRead, kOperandLead, 0);
 #pragma unroll
             for (int i = 0; i < 2 * KSTEPS - kOperandLead; ++i) {
@@ -228,7 +223,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             for (int c4 = 2; c4 < 4; ++c4)
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
-                    vfrag[c4][cb] = lds_read_transposed(&v_lds[buf][v_off + c4 * 16 * VS + cb * 32], VS);
+                    vfrag[c4][cb] = lds_read_transposed_pair(&v_lds[buf][c4 * 16 * D + (t_even ^ (cb << 5))],
+                                                             &v_lds[buf][c4 * 16 * D + (t_odd ^ (cb << 5))]);
 #pragma unroll
             for (int c4 = 0; c4 < 4; ++c4)
 #pragma unroll
@@ -242,10 +238,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        if (more) {
-            kt.store(k_lds[buf ^ 1], k_st);
-            vt.store(v_lds[buf ^ 1], v_st);
-        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's share of the next tile is in LDS
         __syncthreads();
     }
 
