@@ -58,6 +58,47 @@ def test_codes_and_messages_without_a_gpu(lib):
         assert call() == 3 and b"no HIP device" in lib.sentinel_hip_last_error()
 
 
+def test_sparse_rope_and_decode_validation_without_a_gpu(lib):
+    """The newer entry points validate before touching the device, with the reference's message stems."""
+    one = ctypes.c_void_p(16)
+    i, f = ctypes.c_int, ctypes.c_float
+    sparse = lib.sentinel_hip_flash_fwd_sparse
+
+    def call(window=4, global_tokens=0, causal=1, cos=None, sin=None, positions=0):
+        return sparse(one, one, one, one, one, cos, sin, positions, 0, window, global_tokens, 0, -1, 0, 4, 4, 16, 192, 0, 48, 4,
+                      0.25, causal, None, 0, None)
+
+    assert call(global_tokens=-1) == 1 and b"globalTokenCount must be >= 0" in lib.sentinel_hip_last_error()
+    assert call(causal=0) == 1 and b"causal must be set" in lib.sentinel_hip_last_error()
+    assert call(cos=one) == 1 and b"empty tables" in lib.sentinel_hip_last_error()            # one table without the other
+    assert call(cos=one, sin=one, positions=10) == 1 and b"position exceeds RoPE table" in lib.sentinel_hip_last_error()
+    if not lib.sentinel_hip_device_available():
+        assert call() == 3 and b"no HIP device" in lib.sentinel_hip_last_error()
+        assert call(window=0, causal=0) == 3  # no window: the causal flag is free again
+
+    rotate = lib.sentinel_hip_rope_rotate
+    assert rotate(one, 2, 15, 12, 0, 12, 0, 0, one, one, 32, 0, None) == 1 and b"invalid rope dims" in lib.sentinel_hip_last_error()
+    assert rotate(one, 2, 16, 12, 0, 12, 0, 0, one, one, 10, 0, None) == 1 and b"position exceeds RoPE table" in lib.sentinel_hip_last_error()
+    assert rotate(one, 2, 16, 12, 4, 12, 0, 0, one, one, 32, 0, None) == 1 and b"column window outside the matrix" in lib.sentinel_hip_last_error()
+
+    decode = lib.sentinel_hip_decode_attention
+
+    def dec(hq=4, hkv=4, d=16, stride=64, length=20, scale=0.25, window=0, global_tokens=0, ws=one, ws_bytes=1 << 20):
+        return decode(one, one, one, one, hq, hkv, d, stride, length, scale, window, global_tokens, ws, ws_bytes, None)
+
+    assert dec(length=0) == 1 and b"cache is empty" in lib.sentinel_hip_last_error()
+    assert dec(length=65) == 1 and b"cache length exceeds its capacity" in lib.sentinel_hip_last_error()
+    assert dec(hq=6, hkv=4) == 1 and b"divisible by kvHeadCount" in lib.sentinel_hip_last_error()
+    assert dec(hq=12, hkv=4) == 2 and b"must be 1, 2, 4 or 8" in lib.sentinel_hip_last_error()
+    assert dec(d=12) == 2 and b"multiple of 8" in lib.sentinel_hip_last_error()
+    assert dec(global_tokens=-1) == 1 and b"globalTokenCount must be >= 0" in lib.sentinel_hip_last_error()
+    assert dec(ws_bytes=8) == 1 and b"workspace" in lib.sentinel_hip_last_error()
+    need = lib.sentinel_hip_decode_workspace_bytes
+    assert need(4, 16, 20) == 512                             # one chunk of 64 positions, 4 heads, d + 2 floats: 288 B, rounded to 256
+    assert need(32, 128, 32768) == 128 * 32 * 130 * 4         # chunks of 256 positions past 8192 (a multiple of 256 already)
+    assert need(4, 16, 0) == 0
+
+
 def test_workspace_sizes(lib):
     ws = lib.sentinel_hip_flash_workspace_bytes
     assert ws(0, -1, 0, 4, 4, 16, 48, 4, 1) == 0          # fp32 arithmetic needs none
