@@ -703,14 +703,13 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     auto store_stage = [&](DkvSplitStage<D>& st, int it) {
         qtile.store(st.q, st_off);
         gtile.store(st.g, st_off);
-        if (row_thread) {
-            const int q0 = (q_first + it % n_qt) * QT;
-            const bool live = q0 + row_slot < T;
-            if (row_is_delta)
-                st.ndl[stage_slot(row_slot)] = live ? -row_val : 0.0f;
-            else
-                st.nls[stage_slot(row_slot)] = live ? row_val * neg_inv_scale : -__builtin_inff();
-        }
+        // Every thread publishes its row value (threads 128.. repeat the values of threads 0..127): with a branch
+        // around the store the compiler sinks the load into it, to the end of the trip, where its latency holds up
+        // the workgroup barrier.
+        const int q0 = (q_first + it % n_qt) * QT;
+        const bool live = q0 + row_slot < T;
+        float* slot = (row_is_delta ? st.ndl : st.nls) + stage_slot(row_slot);
+        *slot = row_is_delta ? (live ? -row_val : 0.0f) : (live ? row_val * neg_inv_scale : -__builtin_inff());
     };
 
     load_stage(0);
@@ -766,9 +765,9 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     // The next stage's global loads are issued just ahead of the last matrix chain of a trip (no LDS access
     // follows them in the trip) and published to LDS behind it; then every wavefront meets at the barrier.
     // Past the last stage the fetch repeats that stage into the (then unused) next buffer: no branch in a trip.
+    auto prefetch = [&](int it) { load_stage(min(it + 1, n_iter - 1)); };
     auto last_chain = [&](int it, auto&& chain) {
         const int next = min(it + 1, n_iter - 1);
-        load_stage(next);
         chain();
         store_stage(lds.stage[(it + 1) % 3], next);
         __syncthreads();
@@ -801,6 +800,9 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) s = E::mfma(qrow[ks], of[ks], s);
             read_cols(cols + kGOff + blk * 32 * QS, gcol);
+            // the next stage's global loads go out behind the first chain of the trip: their address arithmetic runs
+            // under it and their latency under the rest of the trip
+            if (blk == 0) prefetch(it);
             fence();
             u32x4 pf[2];
 #pragma unroll
@@ -860,6 +862,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
             const u32x4 pf0 = pin[(blk * 2 + 0) * 64];
             const u32x4 pf1 = pin[(blk * 2 + 1) * 64];
             read_cols(cols + blk * 32 * QS, qcol);
+            if (blk == 0) prefetch(it);
             fence();
             u32x4 dsf[2];
 #pragma unroll
@@ -900,6 +903,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         }
         __syncthreads();
     } else {
+        prefetch(0);
         last_chain(0, [] {});
         for (int it = 1; it <= n_iter; ++it) grad_trip(it);
     }

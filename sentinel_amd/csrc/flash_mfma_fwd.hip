@@ -44,8 +44,13 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     constexpr int KSTEPS = D / 16;  // k-steps of the S^T product
     constexpr int CB = D / 32;      // 32-row blocks of O^T
 
-    __shared__ __attribute__((aligned(16))) unsigned short k_lds[2][Tile::kElems];
-    __shared__ __attribute__((aligned(16))) unsigned short v_lds[2][Tile::kElems];
+    // two stages of (K, V) tiles; separate arrays so that the loads streaming into one stage are known not to
+    // alias the operand reads of the other (one array indexed by stage makes the compiler wait for the loads
+    // before every LDS read)
+    __shared__ __attribute__((aligned(16))) unsigned short k_lds0[Tile::kElems];
+    __shared__ __attribute__((aligned(16))) unsigned short v_lds0[Tile::kElems];
+    __shared__ __attribute__((aligned(16))) unsigned short k_lds1[Tile::kElems];
+    __shared__ __attribute__((aligned(16))) unsigned short v_lds1[Tile::kElems];
 
     // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of tiles so
     // that the q-tiles of one head (which stream the same K/V) share one L2.
@@ -95,8 +100,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     const __amdgpu_buffer_rsrc_t k_rsrc = make_head_rsrc(kb, (long long)T * D * 2);
     const __amdgpu_buffer_rsrc_t v_rsrc = make_head_rsrc(vb, (long long)T * D * 2);
     const int ld_off = Tile::global_offset(tid);
-    Tile::issue(k_rsrc, k_lds[0], ld_off, tile_of(0) * KT * D * 2, wave);
-    Tile::issue(v_rsrc, v_lds[0], ld_off, tile_of(0) * KT * D * 2, wave);
+    Tile::issue(k_rsrc, k_lds0, ld_off, tile_of(0) * KT * D * 2, wave);
+    Tile::issue(v_rsrc, v_lds0, ld_off, tile_of(0) * KT * D * 2, wave);
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) pin_loaded(qf[ks]);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the first tiles have landed in LDS
@@ -118,12 +123,13 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     const int t_odd = Tile::transposed_read_base(lane, 1);
     const float raise_after = 8.0f;                // log2 units a row maximum may grow before O is rescaled
 
-    for (int j = 0; j < n_trips; ++j) {
-        const int buf = j & 1;
+    // one trip over the tile held in (k_cur, v_cur); the next tile streams into (k_next, v_next) meanwhile
+    auto tile_trip = [&](int j, const unsigned short* k_cur, const unsigned short* v_cur, unsigned short* k_next,
+                         unsigned short* v_next) __attribute__((always_inline)) {
         const bool more = j + 1 < n_trips;
         if (more) {
-            Tile::issue(k_rsrc, k_lds[buf ^ 1], ld_off, tile_of(j + 1) * KT * D * 2, wave);
-            Tile::issue(v_rsrc, v_lds[buf ^ 1], ld_off, tile_of(j + 1) * KT * D * 2, wave);
+            Tile::issue(k_rsrc, k_next, ld_off, tile_of(j + 1) * KT * D * 2, wave);
+            Tile::issue(v_rsrc, v_next, ld_off, tile_of(j + 1) * KT * D * 2, wave);
         }
 
         const int key0 = tile_of(j) * KT;
@@ -140,7 +146,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
 #pragma unroll
             for (int kbk = 0; kbk < 2; ++kbk)
 #pragma unroll
-                for (int ks = 0; ks < KSTEPS; ++ks) kfrag[kbk][ks] = lds_read128(&k_lds[buf][kbk * 32 * D + (k_off ^ (ks << 4))]);
+                for (int ks = 0; ks < KSTEPS; ++ks) kfrag[kbk][ks] = lds_read128(k_cur + kbk * 32 * D + (k_off ^ (ks << 4)));
 #pragma unroll
             for (int kbk = 0; kbk < 2; ++kbk) {
 #pragma unroll
@@ -152,8 +158,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             for (int c4 = 0; c4 < 2; ++c4)
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
-                    vfrag[c4][cb] = lds_read_transposed_pair(&v_lds[buf][c4 * 16 * D + (t_even ^ (cb << 5))],
-                                                             &v_lds[buf][c4 * 16 * D + (t_odd ^ (cb << 5))]);
+                    vfrag[c4][cb] = lds_read_transposed_pair(v_cur + c4 * 16 * D + (t_even ^ (cb << 5)),
+                                                             v_cur + c4 * 16 * D + (t_odd ^ (cb << 5)));
             __builtin_amdgcn_sched_group_barrier(kSchedDsRead, kOperandLead, 0);
 #pragma unroll
             for (int i = 0; i < 2 * KSTEPS - kOperandLead; ++i) {
@@ -223,8 +229,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             for (int c4 = 2; c4 < 4; ++c4)
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
-                    vfrag[c4][cb] = lds_read_transposed_pair(&v_lds[buf][c4 * 16 * D + (t_even ^ (cb << 5))],
-                                                             &v_lds[buf][c4 * 16 * D + (t_odd ^ (cb << 5))]);
+                    vfrag[c4][cb] = lds_read_transposed_pair(v_cur + c4 * 16 * D + (t_even ^ (cb << 5)),
+                                                             v_cur + c4 * 16 * D + (t_odd ^ (cb << 5)));
 #pragma unroll
             for (int c4 = 0; c4 < 4; ++c4)
 #pragma unroll
@@ -240,6 +246,10 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
 
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's share of the next tile is in LDS
         __syncthreads();
+    };
+    for (int j = 0; j < n_trips; j += 2) {
+        tile_trip(j, k_lds0, v_lds0, k_lds1, v_lds1);
+        if (j + 1 < n_trips) tile_trip(j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
     }
 
     const float l_tot = half_sum(l_run);
