@@ -5,13 +5,13 @@
 //     P = exp(S - LSE),  dP = dO V^T,  dS = P o (dP - D) * scale,
 //     dV = P^T dO,  dK = dS^T Q,  dQ = dS K,          D = rowsum(dO o O)
 // but no atomics and no pre-zeroed outputs: the work is split into
-//   delta_mfma_kernel   D per query;
 //   dkdv_split_kernel   key-outer: a workgroup owns 128 keys of one K/V head; per 32-key block one wavefront
 //                       keeps K (as B operand) and dV^T, a second one V and dK^T, and the query tiles of
 //                       every query head of the group stream through LDS (grouped-query gradients are summed
 //                       in registers, replacing reduceKvHeadGradsInto, CudaCausalSelfAttention.cu:36-44);
 //   dq_mfma_kernel      query-outer: a workgroup owns 128 queries, keeps Q, dO (as B operands) and dQ^T in
-//                       registers and streams K / V tiles through LDS (recomputing S and dP).
+//                       registers and streams K / V tiles through LDS (recomputing S and dP); it runs first and
+//                       also forms D from the dO rows it holds and the O rows, leaving it for the other kernel.
 // Tiles sit row-major in LDS; the products that contract over tokens (dV, dK, dQ) read their A operand out
 // of the same tiles with transposing LDS reads, so nothing is staged twice.
 // In both kernels the score-like tiles are produced so that one lane owns one key (dK/dV kernel) or one
@@ -34,34 +34,6 @@ constexpr int kSchedDsRead = 0x100;
 constexpr int kOperandLead = 4;
 
 // ------------------------------------------------------------------------------------------------
-// D[h][b*T + t] = sum_c out * d_out  (16-bit inputs, fp32 sum)
-// ------------------------------------------------------------------------------------------------
-template <typename E, int D>
-__global__ __launch_bounds__(kBwdThreads) void delta_mfma_kernel(const unsigned short* __restrict__ out,
-                                                                  const unsigned short* __restrict__ d_out,
-                                                                  float* __restrict__ delta, AttnGeom g) {
-    constexpr int LPR = D / 8;  // lanes per row
-    constexpr int RPB = kBwdThreads / LPR;
-    const int tid = threadIdx.x;
-    const int row = blockIdx.x * RPB + tid / LPR;
-    const int part = tid % LPR;
-    const int h = blockIdx.y;
-    const int b = blockIdx.z;
-    const int T = g.seq_len;
-    float sum = 0.0f;
-    if (row < T) {
-        const long long off = (((long long)b * g.q_heads + h) * T + row) * D + part * 8;
-        const u32x4 o = *reinterpret_cast<const u32x4*>(out + off);
-        const u32x4 d = *reinterpret_cast<const u32x4*>(d_out + off);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) sum += E::lo(o[e]) * E::lo(d[e]) + E::hi(o[e]) * E::hi(d[e]);
-    }
-#pragma unroll
-    for (int step = LPR / 2; step >= 1; step /= 2) sum += __shfl_xor(sum, step, LPR);
-    if (part == 0 && row < T) delta[(long long)h * g.packs * T + (long long)b * T + row] = sum;
-}
-
-// ------------------------------------------------------------------------------------------------
 // dQ: query-outer
 // ------------------------------------------------------------------------------------------------
 constexpr int kDqQueryTile = 128;
@@ -71,9 +43,10 @@ template <typename E, int D, bool CAUSAL, bool WINDOW>
 __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned short* __restrict__ q,
                                                                   const unsigned short* __restrict__ k,
                                                                   const unsigned short* __restrict__ v,
+                                                                  const unsigned short* __restrict__ out,
                                                                   const unsigned short* __restrict__ d_out,
                                                                   const float* __restrict__ lse,
-                                                                  const float* __restrict__ delta,
+                                                                  float* __restrict__ delta,
                                                                   unsigned short* __restrict__ dq, RowMap lm, AttnGeom g,
                                                                   int q_tiles, int total_tiles) {
     constexpr int KT = kDqKeyTile;
@@ -120,7 +93,21 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     }
     const float c2 = g.scale * kLog2e;
     const float lse2_raw = lse[b * lm.pack_stride + h * lm.head_stride + qload];
-    float dl = delta[(long long)h * g.packs * T + (long long)b * T + qload];
+    // D = sum_c dO * O of this lane's query: the lane holds half of the row's dO (8 dims per k-step), the other
+    // half sits 32 lanes away.  Computed here (the dO row is in registers anyway) and left in `delta` for the
+    // dK/dV kernel, which runs after this one: no separate pass over O and dO.
+    float dl;
+    {
+        float part = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            const u32x4 o = *reinterpret_cast<const u32x4*>(out + q_head + (long long)qload * D + ks * 16 + gh * 8);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) part += E::lo(o[e]) * E::lo(gf[ks][e]) + E::hi(o[e]) * E::hi(gf[ks][e]);
+        }
+        dl = half_sum(part);
+        if (gh == 0 && qrow < T) delta[(long long)h * g.packs * T + (long long)b * T + qrow] = dl;
+    }
 
     const int q_hi = min(T, (qt + 1) * kDqQueryTile);
     const int kv_tiles = CAUSAL ? (q_hi + KT - 1) / KT : (T + KT - 1) / KT;
@@ -936,16 +923,25 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
     auto dvp = static_cast<unsigned short*>(dv);
     const int T = g.seq_len;
 
-    constexpr int RPB = kBwdThreads / (D / 8);
     hipError_t err;
+    // dQ first: it also leaves D = rowsum(dO o O) in `delta` for the dK/dV kernel
     {
-        KernelTimer timer("delta_mfma", stream);
-        hipLaunchKernelGGL((delta_mfma_kernel<E, D>), dim3((T + RPB - 1) / RPB, g.q_heads, g.packs), dim3(kBwdThreads), 0,
-                           stream, op, gp, delta, g);
+        const int q_tiles = (T + kDqQueryTile - 1) / kDqQueryTile;
+        const int total = g.packs * g.q_heads * q_tiles;
+        const int grid = (total + 7) / 8 * 8;
+        KernelTimer timer("dq_mfma", stream);
+        if (g.window > 0)
+            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true, true>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp,
+                               lse, delta, dqp, lm, g, q_tiles, total);
+        else if (g.causal)
+            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp,
+                               lse, delta, dqp, lm, g, q_tiles, total);
+        else
+            hipLaunchKernelGGL((dq_mfma_kernel<E, D, false, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp,
+                               lse, delta, dqp, lm, g, q_tiles, total);
         err = hipGetLastError();
+        if (err != hipSuccess) return err;
     }
-    if (err != hipSuccess) return err;
-
     // dK, dV
     if constexpr (D <= 64) {
         const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
@@ -991,23 +987,6 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
                                kp, vp, gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
-    }
-    // dQ
-    {
-        const int q_tiles = (T + kDqQueryTile - 1) / kDqQueryTile;
-        const int total = g.packs * g.q_heads * q_tiles;
-        const int grid = (total + 7) / 8 * 8;
-        KernelTimer timer("dq_mfma", stream);
-        if (g.window > 0)
-            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true, true>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp,
-                               lse, delta, dqp, lm, g, q_tiles, total);
-        else if (g.causal)
-            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp,
-                               lse, delta, dqp, lm, g, q_tiles, total);
-        else
-            hipLaunchKernelGGL((dq_mfma_kernel<E, D, false, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, gp,
-                               lse, delta, dqp, lm, g, q_tiles, total);
-        err = hipGetLastError();
     }
     return err;
 }
