@@ -778,8 +778,8 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         u32x4 qrow[KSTEPS];
         u32x4 gcol[2][CB];
         f32x16 s;
+        row_values(nls_off, 0, s);  // first: the chain's first instruction needs the accumulator start and one operand only
         read_rows(rows, qrow);
-        row_values(nls_off, 0, s);
         fence();
 #pragma unroll
         for (int blk = 0; blk < QT / 32; ++blk) {
@@ -838,8 +838,8 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         u32x4 grow[KSTEPS];
         u32x4 qcol[2][CB];
         f32x16 dp;
-        read_rows(rows + kGOff, grow);
         row_values(ndl_off, 0, dp);
+        read_rows(rows + kGOff, grow);
         fence();
 #pragma unroll
         for (int blk = 0; blk < QT / 32; ++blk) {
