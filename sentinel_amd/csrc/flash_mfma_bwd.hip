@@ -369,6 +369,28 @@ __device__ __forceinline__ int dkv_query_tiles(const AttnGeom& g, int k0, int q_
     return q_tiles_all - q_first;
 }
 
+// Workgroup -> (K/V head, key tile).  Workgroup ids are dealt round-robin to the 8 XCDs; each XCD gets a contiguous
+// set of heads (their query tiles stream through one L2).  When the heads divide evenly over the XCDs the key tiles
+// of an XCD's heads are visited tile-major: the first key tiles of every head, which meet the most query tiles
+// (all of them when they hold global tokens of the sparse mask), start together at the head of the grid instead of
+// one head after the other.
+__device__ __forceinline__ bool dkv_tile_of_workgroup(int k_tiles, int total_tiles, int& bkv, int& ktile) {
+    const int per_xcd = (int)gridDim.x / 8;
+    const int xcd = (int)blockIdx.x % 8;
+    const int local = (int)blockIdx.x / 8;
+    const int heads = total_tiles / k_tiles;
+    if (heads % 8 == 0) {
+        const int heads_per_xcd = heads / 8;
+        ktile = local / heads_per_xcd;
+        bkv = xcd * heads_per_xcd + local % heads_per_xcd;
+        return ktile < k_tiles;
+    }
+    const int tile_id = xcd * per_xcd + local;
+    bkv = tile_id / k_tiles;
+    ktile = tile_id % k_tiles;  // under the causal mask the first key tiles see the most queries
+    return tile_id < total_tiles;
+}
+
 template <typename E, int D, bool CAUSAL, bool WINDOW>
 __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
@@ -385,11 +407,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char dkv_smem[];
     DkvLds<D>* lds = reinterpret_cast<DkvLds<D>*>(dkv_smem);  // two stages
 
-    const int per_xcd = (int)gridDim.x / 8;
-    const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
-    if (tile_id >= total_tiles) return;
-    const int bkv = tile_id / k_tiles;
-    const int ktile = tile_id % k_tiles;  // under the causal mask the first key tiles see the most queries
+    int bkv, ktile;
+    if (!dkv_tile_of_workgroup(k_tiles, total_tiles, bkv, ktile)) return;
     const int b = bkv / g.kv_heads;
     const int kvh = bkv % g.kv_heads;
     const int group = g.q_heads / g.kv_heads;
@@ -616,11 +635,8 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char dkv_smem[];
     DkvSplitLds<D>& lds = *reinterpret_cast<DkvSplitLds<D>*>(dkv_smem);
 
-    const int per_xcd = (int)gridDim.x / 8;
-    const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
-    if (tile_id >= total_tiles) return;
-    const int bkv = tile_id / k_tiles;
-    const int ktile = tile_id % k_tiles;
+    int bkv, ktile;
+    if (!dkv_tile_of_workgroup(k_tiles, total_tiles, bkv, ktile)) return;
     const int b = bkv / g.kv_heads;
     const int kvh = bkv % g.kv_heads;
     const int group = g.q_heads / g.kv_heads;
