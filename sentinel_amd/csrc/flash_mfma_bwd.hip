@@ -370,24 +370,34 @@ __device__ __forceinline__ int dkv_query_tiles(const AttnGeom& g, int k0, int q_
 }
 
 // Workgroup -> (K/V head, key tile).  Workgroup ids are dealt round-robin to the 8 XCDs; each XCD gets a contiguous
-// set of heads (their query tiles stream through one L2).  When the heads divide evenly over the XCDs the key tiles
-// of an XCD's heads are visited tile-major: the first key tiles of every head, which meet the most query tiles
-// (all of them when they hold global tokens of the sparse mask), start together at the head of the grid instead of
-// one head after the other.
-__device__ __forceinline__ bool dkv_tile_of_workgroup(int k_tiles, int total_tiles, int& bkv, int& ktile) {
+// set of heads and walks them head after head, key tiles in increasing order: the key tiles of one head run side by
+// side on the XCD and share that head's Q / dO stream in its L2 (HBM reads stay at the algorithmic bytes; a tile-major
+// order over the heads was 2 % faster and read five times as much).  Under the causal mask the first key tiles of a
+// head see the most queries, so each head starts with its longest work.  Key tiles that hold global tokens of the
+// sparse mask (`front_tiles` of them per head) meet every query tile and are far longer than the windowed ones:
+// those are dealt first, for all heads of the XCD, so that they start together at the head of the grid.
+__device__ __forceinline__ bool dkv_tile_of_workgroup(int k_tiles, int total_tiles, int front_tiles, int& bkv, int& ktile) {
     const int per_xcd = (int)gridDim.x / 8;
     const int xcd = (int)blockIdx.x % 8;
     const int local = (int)blockIdx.x / 8;
     const int heads = total_tiles / k_tiles;
-    if (heads % 8 == 0) {
+    if (front_tiles > 0 && heads % 8 == 0) {
         const int heads_per_xcd = heads / 8;
-        ktile = local / heads_per_xcd;
-        bkv = xcd * heads_per_xcd + local % heads_per_xcd;
-        return ktile < k_tiles;
+        const int front = front_tiles * heads_per_xcd;
+        if (local < front) {
+            ktile = local / heads_per_xcd;
+            bkv = xcd * heads_per_xcd + local % heads_per_xcd;
+        } else {
+            const int rest = local - front;
+            const int tail_tiles = k_tiles - front_tiles;
+            bkv = xcd * heads_per_xcd + rest / tail_tiles;
+            ktile = front_tiles + rest % tail_tiles;
+        }
+        return local < per_xcd && bkv < heads;
     }
     const int tile_id = xcd * per_xcd + local;
     bkv = tile_id / k_tiles;
-    ktile = tile_id % k_tiles;  // under the causal mask the first key tiles see the most queries
+    ktile = tile_id % k_tiles;
     return tile_id < total_tiles;
 }
 
@@ -408,7 +418,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     DkvLds<D>* lds = reinterpret_cast<DkvLds<D>*>(dkv_smem);  // two stages
 
     int bkv, ktile;
-    if (!dkv_tile_of_workgroup(k_tiles, total_tiles, bkv, ktile)) return;
+    const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
+    if (!dkv_tile_of_workgroup(k_tiles, total_tiles, front_tiles, bkv, ktile)) return;
     const int b = bkv / g.kv_heads;
     const int kvh = bkv % g.kv_heads;
     const int group = g.q_heads / g.kv_heads;
@@ -636,7 +647,8 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     DkvSplitLds<D>& lds = *reinterpret_cast<DkvSplitLds<D>*>(dkv_smem);
 
     int bkv, ktile;
-    if (!dkv_tile_of_workgroup(k_tiles, total_tiles, bkv, ktile)) return;
+    const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
+    if (!dkv_tile_of_workgroup(k_tiles, total_tiles, front_tiles, bkv, ktile)) return;
     const int b = bkv / g.kv_heads;
     const int kvh = bkv % g.kv_heads;
     const int group = g.q_heads / g.kv_heads;
