@@ -38,7 +38,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
                                                                    const unsigned short* __restrict__ v,
                                                                    unsigned short* __restrict__ out,
                                                                    float* __restrict__ lse, RowMap lm, AttnGeom g,
-                                                                   int q_tiles, int total_tiles) {
+                                                                   int q_tiles, int total_tiles, int tiles_per_xcd) {
     constexpr int KT = kFwdKeyTile;
     typedef DirectTile<KT, D, kFwdThreads> Tile;
     constexpr int KSTEPS = D / 16;  // k-steps of the S^T product
@@ -52,23 +52,31 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     __shared__ __attribute__((aligned(16))) unsigned short k_lds1[Tile::kElems];
     __shared__ __attribute__((aligned(16))) unsigned short v_lds1[Tile::kElems];
 
-    // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of tiles so
-    // that the q-tiles of one head (which stream the same K/V) share one L2.
-    const int per_xcd = (int)gridDim.x / 8;
-    const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
-    if (tile_id >= total_tiles) return;
-    const int bh = tile_id / q_tiles;
-    const int qt = q_tiles - 1 - tile_id % q_tiles;  // longest first within a head
-    const int b = bh / g.q_heads;
-    const int h = bh % g.q_heads;
-    const int kvh = h / (g.q_heads / g.kv_heads);
     const int T = g.seq_len;
-
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);  // wavefront-uniform by construction; tell the compiler
     const int lane = tid % 64;
     const int n = lane % 32;
     const int gh = lane / 32;
+
+    // Persistent workgroups: the grid holds as many workgroups as the device runs at once and each walks several
+    // query tiles (launching a workgroup costs about 5 us of its slot, a sixth of an average tile at T = 4096).
+    // Workgroup ids are dealt round-robin to the 8 XCDs; each XCD owns a contiguous range of tiles (head-major,
+    // longest query tile of a head first), so the query tiles of one head, which stream the same K / V, share one
+    // L2.  Round r hands the XCD's tiles [r S, (r + 1) S) to its S workgroups, forwards in even rounds and backwards
+    // in odd ones: long and short tiles alternate and every workgroup ends up with about the same work.
+    const int xcd = (int)blockIdx.x % 8;
+    const int slot = (int)blockIdx.x / 8;
+    const int slots = (int)gridDim.x / 8;
+    for (int round = 0;; ++round) {
+    const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
+    const int tile_id = xcd * tiles_per_xcd + local_tile;
+    if (local_tile >= tiles_per_xcd || tile_id >= total_tiles) break;
+    const int bh = tile_id / q_tiles;
+    const int qt = q_tiles - 1 - tile_id % q_tiles;  // longest first within a head
+    const int b = bh / g.q_heads;
+    const int h = bh % g.q_heads;
+    const int kvh = h / (g.q_heads / g.kv_heads);
 
     const unsigned short* qb = q + ((long long)b * g.q_heads + h) * T * D;
     const unsigned short* kb = k + ((long long)b * g.kv_heads + kvh) * T * D;
@@ -268,6 +276,20 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
         if (gh == 0)
             lse[b * lm.pack_stride + h * lm.head_stride + qrow] = m_run * g.scale + (l_tot > 0.0f ? __logf(l_tot) : 0.0f);
     }
+    }  // next tile of this workgroup (the last trip ended with a barrier: the LDS stages are free)
+}
+
+// Workgroups the device runs at once, per XCD (8 XCDs): occupancy of the kernel times the compute units of an XCD.
+template <typename Kernel>
+int resident_workgroups_per_xcd(Kernel kernel, int threads, size_t dynamic_lds) {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess || per_cu <= 0) per_cu = 1;
+    int device = 0;
+    int cus = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+        cus <= 0)
+        cus = 256;
+    return per_cu * ((cus + 7) / 8);
 }
 
 template <typename E, int D>
@@ -275,21 +297,24 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
                    hipStream_t stream) {
     const int q_tiles = (g.seq_len + kFwdQueryTile - 1) / kFwdQueryTile;
     const int total = g.packs * g.q_heads * q_tiles;
-    const int grid = (total + 7) / 8 * 8;
+    const int tiles_per_xcd = (total + 7) / 8;
     auto qp = static_cast<const unsigned short*>(q);
     auto kp = static_cast<const unsigned short*>(k);
     auto vp = static_cast<const unsigned short*>(v);
     auto op = static_cast<unsigned short*>(out);
-    KernelTimer timer("fwd_mfma", stream);
+    auto launch = [&](auto kernel) {
+        static const int resident = resident_workgroups_per_xcd(kernel, kFwdThreads, 0);  // per kernel instantiation
+        const int grid = 8 * (tiles_per_xcd < resident ? tiles_per_xcd : resident);
+        KernelTimer timer("fwd_mfma", stream);
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm, g, q_tiles, total,
+                           tiles_per_xcd);
+    };
     if (g.window > 0)
-        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, true, true>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op,
-                           lse, lm, g, q_tiles, total);
+        launch(fwd_mfma_kernel<E, D, true, true>);
     else if (g.causal)
-        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, true, false>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op,
-                           lse, lm, g, q_tiles, total);
+        launch(fwd_mfma_kernel<E, D, true, false>);
     else
-        hipLaunchKernelGGL((fwd_mfma_kernel<E, D, false, false>), dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op,
-                           lse, lm, g, q_tiles, total);
+        launch(fwd_mfma_kernel<E, D, false, false>);
     return hipGetLastError();
 }
 
