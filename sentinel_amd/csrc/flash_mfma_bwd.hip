@@ -48,7 +48,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                                                                   const float* __restrict__ lse,
                                                                   float* __restrict__ delta,
                                                                   unsigned short* __restrict__ dq, RowMap lm, AttnGeom g,
-                                                                  int q_tiles, int total_tiles) {
+                                                                  int q_tiles, int total_tiles, int tiles_per_xcd) {
     constexpr int KT = kDqKeyTile;
     typedef DirectTile<KT, D, kBwdThreads> Tile;
     constexpr int KSTEPS = D / 16;
@@ -60,21 +60,29 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     __shared__ __attribute__((aligned(16))) unsigned short k_lds1[Tile::kElems];
     __shared__ __attribute__((aligned(16))) unsigned short v_lds1[Tile::kElems];
 
-    const int per_xcd = (int)gridDim.x / 8;
-    const int tile_id = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
-    if (tile_id >= total_tiles) return;
-    const int bh = tile_id / q_tiles;
-    const int qt = q_tiles - 1 - tile_id % q_tiles;
-    const int b = bh / g.q_heads;
-    const int h = bh % g.q_heads;
-    const int kvh = h / (g.q_heads / g.kv_heads);
     const int T = g.seq_len;
-
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);  // wavefront-uniform by construction; tell the compiler
     const int lane = tid % 64;
     const int n = lane % 32;
     const int gh = lane / 32;
+
+    // Persistent workgroups: as many as the device runs at once, each walking several query tiles.  Each XCD owns a
+    // contiguous range of tiles (head-major, longest query tile of a head first: the tiles of one head stream the same
+    // K / V through one L2); round r hands the XCD's tiles [r S, (r + 1) S) to its S workgroups, forwards in even
+    // rounds and backwards in odd ones, so long and short tiles alternate.
+    const int xcd = (int)blockIdx.x % 8;
+    const int slot = (int)blockIdx.x / 8;
+    const int slots = (int)gridDim.x / 8;
+    for (int round = 0;; ++round) {
+    const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
+    const int tile_id = xcd * tiles_per_xcd + local_tile;
+    if (local_tile >= tiles_per_xcd || tile_id >= total_tiles) break;
+    const int bh = tile_id / q_tiles;
+    const int qt = q_tiles - 1 - tile_id % q_tiles;
+    const int b = bh / g.q_heads;
+    const int h = bh % g.q_heads;
+    const int kvh = h / (g.q_heads / g.kv_heads);
 
     const long long q_head = ((long long)b * g.q_heads + h) * T * D;
     const unsigned short* kb = k + ((long long)b * g.kv_heads + kvh) * T * D;
@@ -274,6 +282,20 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                 *reinterpret_cast<u32x2*>(dst + cb * 32 + a * 8 + gh * 4) = w;
             }
     }
+    }  // next tile of this workgroup (the last trip ended with a barrier: the LDS stages are free)
+}
+
+// Workgroups the device runs at once, per XCD (8 XCDs): occupancy of the kernel times the compute units of an XCD.
+template <typename Kernel>
+int resident_workgroups_per_xcd(Kernel kernel, int threads, size_t dynamic_lds) {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess || per_cu <= 0) per_cu = 1;
+    int device = 0;
+    int cus = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+        cus <= 0)
+        cus = 256;
+    return per_cu * ((cus + 7) / 8);
 }
 
 constexpr int kDkvKeyTile = 128;
@@ -369,17 +391,15 @@ __device__ __forceinline__ int dkv_query_tiles(const AttnGeom& g, int k0, int q_
     return q_tiles_all - q_first;
 }
 
-// Workgroup -> (K/V head, key tile).  Workgroup ids are dealt round-robin to the 8 XCDs; each XCD gets a contiguous
+// Tile `local` of XCD `xcd` -> (K/V head, key tile).  Workgroup ids are dealt round-robin to the 8 XCDs; each XCD gets a contiguous
 // set of heads and walks them head after head, key tiles in increasing order: the key tiles of one head run side by
 // side on the XCD and share that head's Q / dO stream in its L2 (HBM reads stay at the algorithmic bytes; a tile-major
 // order over the heads was 2 % faster and read five times as much).  Under the causal mask the first key tiles of a
 // head see the most queries, so each head starts with its longest work.  Key tiles that hold global tokens of the
 // sparse mask (`front_tiles` of them per head) meet every query tile and are far longer than the windowed ones:
 // those are dealt first, for all heads of the XCD, so that they start together at the head of the grid.
-__device__ __forceinline__ bool dkv_tile_of_workgroup(int k_tiles, int total_tiles, int front_tiles, int& bkv, int& ktile) {
-    const int per_xcd = (int)gridDim.x / 8;
-    const int xcd = (int)blockIdx.x % 8;
-    const int local = (int)blockIdx.x / 8;
+__device__ __forceinline__ bool dkv_tile_of_workgroup(int xcd, int local, int per_xcd, int k_tiles, int total_tiles,
+                                                      int front_tiles, int& bkv, int& ktile) {
     const int heads = total_tiles / k_tiles;
     if (front_tiles > 0 && heads % 8 == 0) {
         const int heads_per_xcd = heads / 8;
@@ -406,7 +426,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
-    int total_tiles) {
+    int total_tiles, int tiles_per_xcd) {
     constexpr int QT = kDkvQueryTile;
     typedef RowTile<QT, D, kBwdThreads, DkvLds<D>::kPad> RTile;
     constexpr int QS = RTile::kStride;
@@ -417,19 +437,27 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char dkv_smem[];
     DkvLds<D>* lds = reinterpret_cast<DkvLds<D>*>(dkv_smem);  // two stages
 
-    int bkv, ktile;
-    const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
-    if (!dkv_tile_of_workgroup(k_tiles, total_tiles, front_tiles, bkv, ktile)) return;
-    const int b = bkv / g.kv_heads;
-    const int kvh = bkv % g.kv_heads;
     const int group = g.q_heads / g.kv_heads;
     const int T = g.seq_len;
-
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);  // wavefront-uniform by construction; tell the compiler
     const int lane = tid % 64;
     const int n = lane % 32;
     const int gh = lane / 32;
+
+    // persistent workgroups walking the XCD's key tiles in snake order (see dq_mfma_kernel)
+    const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
+    const int xcd = (int)blockIdx.x % 8;
+    const int slot = (int)blockIdx.x / 8;
+    const int slots = (int)gridDim.x / 8;
+    for (int round = 0;; ++round) {
+    const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
+    int bkv, ktile;
+    if (local_tile >= tiles_per_xcd ||
+        !dkv_tile_of_workgroup(xcd, local_tile, tiles_per_xcd, k_tiles, total_tiles, front_tiles, bkv, ktile))
+        break;
+    const int b = bkv / g.kv_heads;
+    const int kvh = bkv % g.kv_heads;
 
     const long long kv_head = ((long long)b * g.kv_heads + kvh) * T * D;
     const int k0w = ktile * kDkvKeyTile + wave * 32;
@@ -628,6 +656,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
                 *reinterpret_cast<u32x2*>(dvp + cb * 32 + a * 8 + gh * 4) = wv;
             }
     }
+    }  // next key tile of this workgroup (every stage trip ended with a barrier: the LDS stages are free)
 }
 
 template <typename E, int D, bool CAUSAL, bool WINDOW>
@@ -635,7 +664,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
-    int total_tiles) {
+    int total_tiles, int tiles_per_xcd) {
     constexpr int QT = kDkvQueryTile;
     typedef RowTile<QT, D, kDkvSplitThreads, 8> RTile;
     constexpr int QS = RTile::kStride;
@@ -646,14 +675,8 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char dkv_smem[];
     DkvSplitLds<D>& lds = *reinterpret_cast<DkvSplitLds<D>*>(dkv_smem);
 
-    int bkv, ktile;
-    const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
-    if (!dkv_tile_of_workgroup(k_tiles, total_tiles, front_tiles, bkv, ktile)) return;
-    const int b = bkv / g.kv_heads;
-    const int kvh = bkv % g.kv_heads;
     const int group = g.q_heads / g.kv_heads;
     const int T = g.seq_len;
-
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const bool grad_role = wave >= 4;
@@ -661,6 +684,20 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const int lane = tid % 64;
     const int n = lane % 32;
     const int gh = lane / 32;
+
+    // persistent workgroups walking the XCD's key tiles in snake order (see dq_mfma_kernel)
+    const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
+    const int xcd = (int)blockIdx.x % 8;
+    const int slot = (int)blockIdx.x / 8;
+    const int slots = (int)gridDim.x / 8;
+    for (int round = 0;; ++round) {
+    const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
+    int bkv, ktile;
+    if (local_tile >= tiles_per_xcd ||
+        !dkv_tile_of_workgroup(xcd, local_tile, tiles_per_xcd, k_tiles, total_tiles, front_tiles, bkv, ktile))
+        break;
+    const int b = bkv / g.kv_heads;
+    const int kvh = bkv % g.kv_heads;
 
     const long long kv_head = ((long long)b * g.kv_heads + kvh) * T * D;
     const int k0w = ktile * kDkvKeyTile + kblock * 32;
@@ -936,6 +973,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
                 *reinterpret_cast<u32x2*>(dst + cb * 32 + a * 8 + gh * 4) = w;
             }
     }
+    }  // next key tile of this workgroup (both roles have passed the last barrier of the tile: the LDS is free)
 }
 
 template <typename E, int D>
@@ -956,65 +994,67 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
     {
         const int q_tiles = (T + kDqQueryTile - 1) / kDqQueryTile;
         const int total = g.packs * g.q_heads * q_tiles;
-        const int grid = (total + 7) / 8 * 8;
-        KernelTimer timer("dq_mfma", stream);
+        const int tiles_per_xcd = (total + 7) / 8;
+        auto launch = [&](auto kernel) {
+            static const int resident = resident_workgroups_per_xcd(kernel, kBwdThreads, 0);  // per kernel instantiation
+            const int grid = 8 * (tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            KernelTimer timer("dq_mfma", stream);
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp, lse, delta, dqp, lm, g,
+                               q_tiles, total, tiles_per_xcd);
+        };
         if (g.window > 0)
-            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true, true>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp,
-                               lse, delta, dqp, lm, g, q_tiles, total);
+            launch(dq_mfma_kernel<E, D, true, true>);
         else if (g.causal)
-            hipLaunchKernelGGL((dq_mfma_kernel<E, D, true, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp,
-                               lse, delta, dqp, lm, g, q_tiles, total);
+            launch(dq_mfma_kernel<E, D, true, false>);
         else
-            hipLaunchKernelGGL((dq_mfma_kernel<E, D, false, false>), dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp,
-                               lse, delta, dqp, lm, g, q_tiles, total);
+            launch(dq_mfma_kernel<E, D, false, false>);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
     // dK, dV
+    const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
+    const int total = g.packs * g.kv_heads * k_tiles;
+    const int tiles_per_xcd = (total + 7) / 8;
     if constexpr (D <= 64) {
-        const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
-        const int total = g.packs * g.kv_heads * k_tiles;
-        const int grid = (total + 7) / 8 * 8;
         const size_t smem = 2 * sizeof(DkvLds<D>);
-        KernelTimer timer("dkdv_mfma", stream);
+        auto launch = [&](auto kernel) {
+            static const int resident = resident_workgroups_per_xcd(kernel, kBwdThreads, smem);  // per kernel instantiation
+            // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
+            // dispatched in order (long ones first), balances better than a fixed assignment
+            const int grid = 8 * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            KernelTimer timer("dkdv_mfma", stream);
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp, dvp, lm, g,
+                               k_tiles, total, tiles_per_xcd);
+        };
         if (g.window > 0)
-            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, true, true>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp,
-                               gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
+            launch(dkdv_mfma_kernel<E, D, true, true>);
         else if (g.causal)
-            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, true, false>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp,
-                               gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
+            launch(dkdv_mfma_kernel<E, D, true, false>);
         else
-            hipLaunchKernelGGL((dkdv_mfma_kernel<E, D, false, false>), dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp,
-                               vp, gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
+            launch(dkdv_mfma_kernel<E, D, false, false>);
         err = hipGetLastError();
-        if (err != hipSuccess) return err;
     } else {
-        const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
-        const int total = g.packs * g.kv_heads * k_tiles;
-        const int grid = (total + 7) / 8 * 8;
         const size_t smem = sizeof(DkvSplitLds<D>);
-        static bool raised[3] = {false, false, false};  // one-time opt-in to more than 64 KiB of LDS per kernel
-        const int which = g.window > 0 ? 2 : g.causal ? 1 : 0;
-        if (!raised[which]) {
-            const void* fn = which == 2   ? reinterpret_cast<const void*>(dkdv_split_kernel<E, D, true, true>)
-                             : which == 1 ? reinterpret_cast<const void*>(dkdv_split_kernel<E, D, true, false>)
-                                          : reinterpret_cast<const void*>(dkdv_split_kernel<E, D, false, false>);
-            err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-            if (err != hipSuccess) return err;
-            raised[which] = true;
-        }
-        KernelTimer timer("dkdv_mfma", stream);
-        if (which == 2)
-            hipLaunchKernelGGL((dkdv_split_kernel<E, D, true, true>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp,
-                               kp, vp, gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
-        else if (which == 1)
-            hipLaunchKernelGGL((dkdv_split_kernel<E, D, true, false>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp,
-                               kp, vp, gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
+        auto launch = [&](auto kernel) -> hipError_t {
+            // one-time per kernel instantiation: opt in to more than 64 KiB of LDS, then ask how many workgroups fit
+            static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+            if (raised != hipSuccess) return raised;
+            static const int resident = resident_workgroups_per_xcd(kernel, kDkvSplitThreads, smem);
+            // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
+            // dispatched in order (long ones first), balances better than a fixed assignment
+            const int grid = 8 * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            KernelTimer timer("dkdv_mfma", stream);
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp, dvp, lm, g,
+                               k_tiles, total, tiles_per_xcd);
+            return hipGetLastError();
+        };
+        if (g.window > 0)
+            err = launch(dkdv_split_kernel<E, D, true, true>);
+        else if (g.causal)
+            err = launch(dkdv_split_kernel<E, D, true, false>);
         else
-            hipLaunchKernelGGL((dkdv_split_kernel<E, D, false, false>), dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp,
-                               kp, vp, gp, lse, delta, dkp, dvp, lm, g, k_tiles, total);
-        err = hipGetLastError();
-        if (err != hipSuccess) return err;
+            err = launch(dkdv_split_kernel<E, D, false, false>);
     }
     return err;
 }
