@@ -666,7 +666,9 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
     int total_tiles, int tiles_per_xcd) {
     constexpr int QT = kDkvQueryTile;
-    typedef RowTile<QT, D, kDkvSplitThreads, 8> RTile;
+    // the query / dO tiles of a stage are staged by the score wavefronts alone (threads 0..255): they have about a
+    // quarter of a stage to spare, the grad wavefronts are the critical path
+    typedef RowTile<QT, D, kDkvSplitThreads / 2, 8> RTile;
     constexpr int QS = RTile::kStride;
     static_assert(QS == DkvSplitStage<D>::QS, "LDS layout mismatch");
     constexpr int KSTEPS = D / 16;
@@ -764,8 +766,10 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         *slot = row_is_delta ? (live ? -row_val : 0.0f) : (live ? row_val * neg_inv_scale : -__builtin_inff());
     };
 
-    load_stage(0);
-    store_stage(lds.stage[0], 0);
+    if (!grad_role) {
+        load_stage(0);
+        store_stage(lds.stage[0], 0);
+    }
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) pin_loaded(of[ks]);
     __syncthreads();
@@ -822,6 +826,10 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         const int next = min(it + 1, n_iter - 1);
         chain();
         store_stage(lds.stage[(it + 1) % 3], next);
+        __syncthreads();
+    };
+    auto last_chain_grad = [&](auto&& chain) {
+        chain();
         __syncthreads();
     };
 
@@ -914,7 +922,6 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
             const u32x4 pf0 = pin[(blk * 2 + 0) * 64];
             const u32x4 pf1 = pin[(blk * 2 + 1) * 64];
             read_cols(cols + blk * 32 * QS, qcol);
-            if (blk == 0) prefetch(it);
             fence();
             u32x4 dsf[2];
 #pragma unroll
@@ -936,7 +943,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
                 fence();
             } else {
                 fence();
-                last_chain(it, dk_chain);
+                last_chain_grad(dk_chain);
             }
         }
     };
@@ -955,8 +962,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         }
         __syncthreads();
     } else {
-        prefetch(0);
-        last_chain(0, [] {});
+        __syncthreads();  // trip 0: the score wavefronts work on stage 0 and publish stage 1
         for (int it = 1; it <= n_iter; ++it) grad_trip(it);
     }
 
