@@ -1003,7 +1003,9 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
         const int tiles_per_xcd = (total + 7) / 8;
         auto launch = [&](auto kernel) {
             static const int resident = resident_workgroups_per_xcd(kernel, kBwdThreads, 0);  // per kernel instantiation
-            const int grid = 8 * (tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            // under the sparse mask tile lengths no longer grow with the tile index, and one workgroup per tile handed out
+            // as slots free up is 6 - 13 % faster than the fixed snake assignment
+            const int grid = 8 * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
             KernelTimer timer("dq_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp, lse, delta, dqp, lm, g,
                                q_tiles, total, tiles_per_xcd);
