@@ -270,18 +270,10 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
         if (j + 1 < n_trips) tile_trip(std::true_type{}, j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
     }
 
-    if (qrow < T) {
-        unsigned short* dst = dq + q_head + (long long)qrow * D;
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                u32x2 w;
-                w[0] = E::pack2(acc[cb][a * 4 + 0] * g.scale, acc[cb][a * 4 + 1] * g.scale);
-                w[1] = E::pack2(acc[cb][a * 4 + 2] * g.scale, acc[cb][a * 4 + 3] * g.scale);
-                *reinterpret_cast<u32x2*>(dst + cb * 32 + a * 8 + gh * 4) = w;
-            }
-    }
+    // dQ rows leave through the second LDS stage, which no wavefront reads or fills any more: the last trip ended with
+    // a barrier, and the next tile's first loads go to stage 0 and are followed by a barrier before stage 1 is filled
+    store_rows_via_lds<E, D>(acc, g.scale, (wave < 2 ? k_lds1 : v_lds1) + (wave & 1) * (32 * D),
+                             dq + q_head + (long long)q0w * D, T - q0w, lane);
     }  // next tile of this workgroup (the last trip ended with a barrier: the LDS stages are free)
 }
 
@@ -640,21 +632,14 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
         }
     }
 
-    if (!key_dead) {
-        unsigned short* dkp = dk + kv_head + (long long)key * D;
-        unsigned short* dvp = dv + kv_head + (long long)key * D;
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                u32x2 wk, wv;
-                wk[0] = E::pack2(dk_acc[cb][a * 4 + 0] * g.scale, dk_acc[cb][a * 4 + 1] * g.scale);
-                wk[1] = E::pack2(dk_acc[cb][a * 4 + 2] * g.scale, dk_acc[cb][a * 4 + 3] * g.scale);
-                wv[0] = E::pack2(dv_acc[cb][a * 4 + 0], dv_acc[cb][a * 4 + 1]);
-                wv[1] = E::pack2(dv_acc[cb][a * 4 + 2], dv_acc[cb][a * 4 + 3]);
-                *reinterpret_cast<u32x2*>(dkp + cb * 32 + a * 8 + gh * 4) = wk;
-                *reinterpret_cast<u32x2*>(dvp + cb * 32 + a * 8 + gh * 4) = wv;
-            }
+    {
+        // dK and dV rows leave through the second LDS stage (free: every trip ended with a barrier, and the next key
+        // tile fills stage 0 and passes a barrier before it touches stage 1), one after the other through the same area
+        static_assert(sizeof(DkvLds<D>) >= 4 * 32 * D * 2, "second stage too small to stage the result rows");
+        unsigned short* area = reinterpret_cast<unsigned short*>(&lds[1]) + wave * (32 * D);
+        store_rows_via_lds<E, D>(dk_acc, g.scale, area, dk + kv_head + (long long)k0w * D, T - k0w, lane);
+        __builtin_amdgcn_wave_barrier();
+        store_rows_via_lds<E, D>(dv_acc, 1.0f, area, dv + kv_head + (long long)k0w * D, T - k0w, lane);
     }
     }  // next key tile of this workgroup (every stage trip ended with a barrier: the LDS stages are free)
 }
@@ -966,18 +951,13 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         for (int it = 1; it <= n_iter; ++it) grad_trip(it);
     }
 
-    if (!key_dead) {
-        unsigned short* dst = (grad_role ? dk : dv) + kv_head + (long long)key * D;
-        const float out_scale = grad_role ? g.scale : 1.0f;
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                u32x2 w;
-                w[0] = E::pack2(acc[cb][a * 4 + 0] * out_scale, acc[cb][a * 4 + 1] * out_scale);
-                w[1] = E::pack2(acc[cb][a * 4 + 2] * out_scale, acc[cb][a * 4 + 3] * out_scale);
-                *reinterpret_cast<u32x2*>(dst + cb * 32 + a * 8 + gh * 4) = w;
-            }
+    {
+        // dV (score role) and dK (grad role) rows leave through stages 1 and 2 of the LDS: both roles have passed the
+        // last barrier of the tile, and the next key tile fills stage 0 and passes a barrier before it touches the others
+        static_assert(2 * sizeof(DkvSplitStage<D>) >= 8 * 32 * D * 2, "stages 1 and 2 too small to stage the result rows");
+        unsigned short* area = reinterpret_cast<unsigned short*>(dkv_smem + sizeof(DkvSplitStage<D>)) + wave * (32 * D);
+        store_rows_via_lds<E, D>(acc, grad_role ? g.scale : 1.0f, area,
+                                 (grad_role ? dk : dv) + kv_head + (long long)k0w * D, T - k0w, lane);
     }
     }  // next key tile of this workgroup (both roles have passed the last barrier of the tile: the LDS is free)
 }

@@ -262,20 +262,12 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
 
     const float l_tot = half_sum(l_run);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-    if (qrow < T) {
-        unsigned short* op = out + ((long long)b * g.q_heads + h) * T * D + (long long)qrow * D;
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                u32x2 w;
-                w[0] = E::pack2(acc[cb][a * 4 + 0] * inv, acc[cb][a * 4 + 1] * inv);
-                w[1] = E::pack2(acc[cb][a * 4 + 2] * inv, acc[cb][a * 4 + 3] * inv);
-                *reinterpret_cast<u32x2*>(op + cb * 32 + a * 8 + gh * 4) = w;
-            }
-        if (gh == 0)
-            lse[b * lm.pack_stride + h * lm.head_stride + qrow] = m_run * g.scale + (l_tot > 0.0f ? __logf(l_tot) : 0.0f);
-    }
+    // O rows leave through the second LDS stage, which no wavefront reads or fills any more: the last trip ended with a
+    // barrier, and the next tile's first loads go to stage 0 and are followed by a barrier before stage 1 is filled
+    store_rows_via_lds<E, D, false>(acc, inv, (wave < 2 ? k_lds1 : v_lds1) + (wave & 1) * (32 * D),
+                             out + ((long long)b * g.q_heads + h) * T * D + (long long)q0w * D, T - q0w, lane);
+    if (qrow < T && gh == 0)
+        lse[b * lm.pack_stride + h * lm.head_stride + qrow] = m_run * g.scale + (l_tot > 0.0f ? __logf(l_tot) : 0.0f);
     }  // next tile of this workgroup (the last trip ended with a barrier: the LDS stages are free)
 }
 
