@@ -71,6 +71,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     // contiguous range of tiles (head-major, longest query tile of a head first: the tiles of one head stream the same
     // K / V through one L2); round r hands the XCD's tiles [r S, (r + 1) S) to its S workgroups, forwards in even
     // rounds and backwards in odd ones, so long and short tiles alternate.
+    const unsigned turn_class = priority_turn_class();
     const int xcd = (int)blockIdx.x % 8;
     const int slot = (int)blockIdx.x / 8;
     const int slots = (int)gridDim.x / 8;
@@ -253,8 +254,10 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        const unsigned now = WINDOW ? 0u : (unsigned)__builtin_amdgcn_s_memrealtime();
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's share of the next tile is in LDS
         __syncthreads();
+        if (!WINDOW) take_priority_turn(now, turn_class);  // the persistent grid only: see take_priority_turn
     };
 
     // Tiles that end at or before the first query of the workgroup need no mask for any wavefront; keep the count

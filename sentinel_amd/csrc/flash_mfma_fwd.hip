@@ -65,6 +65,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     // longest query tile of a head first), so the query tiles of one head, which stream the same K / V, share one
     // L2.  Round r hands the XCD's tiles [r S, (r + 1) S) to its S workgroups, forwards in even rounds and backwards
     // in odd ones: long and short tiles alternate and every workgroup ends up with about the same work.
+    const unsigned turn_class = priority_turn_class();
     const int xcd = (int)blockIdx.x % 8;
     const int slot = (int)blockIdx.x / 8;
     const int slots = (int)gridDim.x / 8;
@@ -252,8 +253,10 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             __builtin_amdgcn_sched_barrier(0);
         }
 
+        const unsigned now = WINDOW ? 0u : (unsigned)__builtin_amdgcn_s_memrealtime();
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's share of the next tile is in LDS
         __syncthreads();
+        if (!WINDOW) take_priority_turn(now, turn_class);  // the persistent grid only: see take_priority_turn
     };
     for (int j = 0; j < n_trips; j += 2) {
         tile_trip(j, k_lds0, v_lds0, k_lds1, v_lds1);

@@ -235,6 +235,21 @@ __device__ __forceinline__ u32x4 lds_read_transposed_pair(const unsigned short* 
 }
 
 
+// Two workgroups share a compute unit, one wavefront of each per SIMD, and the hardware issues the older wavefront first
+// whenever both are ready: the workgroup that arrived first runs about 1.6 times as fast as the other and finishes its
+// tiles early, after which the compute unit is half empty.  Taking turns at the higher priority (the turn changes every
+// 2^13 ticks of the constant 100 MHz clock, 82 us; which of the two starts is decided by the wavefront's slot on its SIMD)
+// evens the two out, so all workgroups of the persistent grid finish together.
+__device__ __forceinline__ unsigned priority_turn_class() {
+    return __builtin_amdgcn_s_getreg((3 << 11) | 4) & 1u;  // HW_ID.wave_id, bit 0
+}
+__device__ __forceinline__ void take_priority_turn(unsigned realtime, unsigned turn_class) {
+    if (((realtime >> 13) ^ turn_class) & 1u)
+        __builtin_amdgcn_s_setprio(1);
+    else
+        __builtin_amdgcn_s_setprio(0);
+}
+
 // Writes a wavefront's 32 x D block of 16-bit results to 32 consecutive global rows of D elements.  The block is held as
 // transposed accumulators: lane (n, gh) owns row n, elements cb*32 + a*8 + gh*4 + [0, 4) in acc[cb][a*4 + ...].  Stored
 // straight from there, one instruction would write 16 bytes to each of 32 rows (64 partial-line requests); passing
