@@ -253,10 +253,12 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        const unsigned now = WINDOW ? 0u : (unsigned)__builtin_amdgcn_s_memrealtime();
+        // priority turns: for the persistent grid with two workgroups per compute unit (head_dim 128) only
+        constexpr bool TURNS = !WINDOW && D > 64;
+        const unsigned now = TURNS ? (unsigned)__builtin_amdgcn_s_memrealtime() : 0u;
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's share of the next tile is in LDS
         __syncthreads();
-        if (!WINDOW) take_priority_turn(now, turn_class);  // the persistent grid only: see take_priority_turn
+        if (TURNS) take_priority_turn(now, turn_class);
     };
     for (int j = 0; j < n_trips; j += 2) {
         tile_trip(j, k_lds0, v_lds0, k_lds1, v_lds1);
