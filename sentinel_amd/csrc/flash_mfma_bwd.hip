@@ -948,19 +948,25 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
             if (WINDOW)
                 for (; it < head_end; ++it) score_trip(std::true_type{}, it);
         }
+        // Last trip of the tile: the grad wavefronts work on the last stage, the score wavefronts have none left and
+        // store dV meanwhile.  The stage buffers are still in use; the rows pass through the P buffer this trip would
+        // have filled, 4 KB per wavefront, 16 rows at a time.
+        static_assert(kPBufBytes >= 4 * 16 * D * 2, "P buffer too small to stage the dV rows");
+        store_rows_via_lds<E, D, true, 16>(
+            acc, 1.0f, reinterpret_cast<unsigned short*>(dkv_smem + kPBase + (n_iter & 1) * kPBufBytes) + kblock * (16 * D),
+            dv + kv_head + (long long)k0w * D, T - k0w, lane);
         __syncthreads();
     } else {
         __syncthreads();  // trip 0: the score wavefronts work on stage 0 and publish stage 1
         for (int it = 1; it <= n_iter; ++it) grad_trip(it);
     }
 
-    {
-        // dV (score role) and dK (grad role) rows leave through stages 1 and 2 of the LDS: both roles have passed the
-        // last barrier of the tile, and the next key tile fills stage 0 and passes a barrier before it touches the others
-        static_assert(2 * sizeof(DkvSplitStage<D>) >= 8 * 32 * D * 2, "stages 1 and 2 too small to stage the result rows");
-        unsigned short* area = reinterpret_cast<unsigned short*>(dkv_smem + sizeof(DkvSplitStage<D>)) + wave * (32 * D);
-        store_rows_via_lds<E, D>(acc, grad_role ? g.scale : 1.0f, area,
-                                 (grad_role ? dk : dv) + kv_head + (long long)k0w * D, T - k0w, lane);
+    if (grad_role) {
+        // dK rows leave through stages 1 and 2 of the LDS: both roles have passed the last barrier of the tile, and the
+        // next key tile fills stage 0 and passes a barrier before it touches the others
+        static_assert(2 * sizeof(DkvSplitStage<D>) >= 4 * 32 * D * 2, "stages 1 and 2 too small to stage the dK rows");
+        unsigned short* area = reinterpret_cast<unsigned short*>(dkv_smem + sizeof(DkvSplitStage<D>)) + kblock * (32 * D);
+        store_rows_via_lds<E, D>(acc, g.scale, area, dk + kv_head + (long long)k0w * D, T - k0w, lane);
     }
     }  // next key tile of this workgroup (both roles have passed the last barrier of the tile: the LDS is free)
 }

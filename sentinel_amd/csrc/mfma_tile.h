@@ -253,37 +253,48 @@ __device__ __forceinline__ void take_priority_turn(unsigned realtime, unsigned t
 // Writes a wavefront's 32 x D block of 16-bit results to 32 consecutive global rows of D elements.  The block is held as
 // transposed accumulators: lane (n, gh) owns row n, elements cb*32 + a*8 + gh*4 + [0, 4) in acc[cb][a*4 + ...].  Stored
 // straight from there, one instruction would write 16 bytes to each of 32 rows (64 partial-line requests); passing
-// through a wavefront-private LDS area (32 * D elements) turns that into whole 16 * D-byte runs per instruction.  16-byte
+// through a wavefront-private LDS area (ROWS_PER_PASS * D elements) turns that into whole 16 * D-byte runs per
+// instruction.  16-byte
 // pieces of a row are XOR-swizzled with the row number to spread the column-wise writes over the banks.  LDS
 // instructions of one wavefront execute in order, so no wait is needed between the writes and the reads.
 // PIN_ADDRESSES keeps the per-lane address arithmetic at the call site: hoisted over the caller's loops it costs about
 // twenty registers there, which the kernels that already use all 256 pay for with spills.
-template <class E, int D, bool PIN_ADDRESSES = true>
+template <class E, int D, bool PIN_ADDRESSES = true, int ROWS_PER_PASS = 32>
 __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], float factor, unsigned short* lds,
                                                    unsigned short* dst, int valid_rows, int lane) {
     constexpr int PIECES = D / 8;          // 16-byte pieces per row
     constexpr int ROWS_PER_STORE = 64 / PIECES;
+    static_assert(32 % ROWS_PER_PASS == 0 && ROWS_PER_PASS % ROWS_PER_STORE == 0, "pass / store shape mismatch");
     if (PIN_ADDRESSES) asm volatile("" : "+v"(lane));
     const int n = lane % 32;
     const int gh = lane / 32;
     unsigned char* base = reinterpret_cast<unsigned char*>(lds);
-#pragma unroll
-    for (int cb = 0; cb < D / 32; ++cb)
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-            u32x2 w;
-            w[0] = E::pack2(acc[cb][a * 4 + 0] * factor, acc[cb][a * 4 + 1] * factor);
-            w[1] = E::pack2(acc[cb][a * 4 + 2] * factor, acc[cb][a * 4 + 3] * factor);
-            const int piece = cb * 4 + a;
-            *reinterpret_cast<u32x2*>(base + n * (D * 2) + ((piece ^ (n & (PIECES - 1))) << 4) + gh * 8) = w;
-        }
-    __builtin_amdgcn_wave_barrier();
     const int p = lane % PIECES;
+    // with ROWS_PER_PASS < 32 the area holds ROWS_PER_PASS * D elements and the block goes through it in several passes
 #pragma unroll
-    for (int i = 0; i < 32 / ROWS_PER_STORE; ++i) {
-        const int r = i * ROWS_PER_STORE + lane / PIECES;
-        const u32x4 val = *reinterpret_cast<const u32x4*>(base + r * (D * 2) + ((p ^ (r & (PIECES - 1))) << 4));
-        if (r < valid_rows) *reinterpret_cast<u32x4*>(dst + (long long)r * D + p * 8) = val;
+    for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
+        if (ROWS_PER_PASS == 32 || n / ROWS_PER_PASS == pass) {
+            const int row = n % ROWS_PER_PASS;
+#pragma unroll
+            for (int cb = 0; cb < D / 32; ++cb)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    u32x2 w;
+                    w[0] = E::pack2(acc[cb][a * 4 + 0] * factor, acc[cb][a * 4 + 1] * factor);
+                    w[1] = E::pack2(acc[cb][a * 4 + 2] * factor, acc[cb][a * 4 + 3] * factor);
+                    const int piece = cb * 4 + a;
+                    *reinterpret_cast<u32x2*>(base + row * (D * 2) + ((piece ^ (row & (PIECES - 1))) << 4) + gh * 8) = w;
+                }
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < ROWS_PER_PASS / ROWS_PER_STORE; ++i) {
+            const int r = i * ROWS_PER_STORE + lane / PIECES;
+            const u32x4 val = *reinterpret_cast<const u32x4*>(base + r * (D * 2) + ((p ^ (r & (PIECES - 1))) << 4));
+            const int out_row = pass * ROWS_PER_PASS + r;
+            if (out_row < valid_rows) *reinterpret_cast<u32x4*>(dst + (long long)out_row * D + p * 8) = val;
+        }
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
