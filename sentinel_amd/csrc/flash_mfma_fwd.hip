@@ -6,7 +6,7 @@
 //     a loop-invariant vector offset (the hardware range check zero-fills rows past T); nothing is
 //     converted or gathered per tile;
 //   * a workgroup of 4 wavefronts owns 128 queries (32 per wavefront) and walks 64-key tiles;
-//     Q stays in registers for the whole kernel, K and V tiles are double-buffered in LDS (row-major,
+//     Q stays in registers for the whole query tile, K and V tiles are double-buffered in LDS (row-major,
 //     XOR-swizzled) and the next tile streams straight into LDS (buffer_load ... lds) while the current one
 //     is multiplied;
 //   * S^T = K Q^T, so a lane owns one query: the online-softmax max / sum are in-register plus one
@@ -16,7 +16,9 @@
 //     which is exact and keeps P within the 16-bit range;
 //   * key tiles above the diagonal are skipped; only tiles that cross it are masked; with Sentinel's sparse mask
 //     (sliding window + global tokens, WINDOW) the key tiles below every window of the query tile are skipped too;
-//   * grouped-query attention reads the shared K/V head in place.
+//   * grouped-query attention reads the shared K/V head in place;
+//   * the grid is persistent (as many workgroups as the device runs at once, each walking several query tiles), the two
+//     workgroups of a compute unit take turns at the higher wave priority, and the O rows leave through LDS as whole rows.
 #include "flash_common.h"
 #include "mfma_tile.h"
 
