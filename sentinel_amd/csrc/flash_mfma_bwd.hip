@@ -442,6 +442,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
 
     // persistent workgroups walking the XCD's key tiles in snake order (see dq_mfma_kernel)
     const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
+    const unsigned turn_class = priority_turn_class();
     const int xcd = (int)blockIdx.x % 8;
     const int slot = (int)blockIdx.x / 8;
     const int slots = (int)gridDim.x / 8;
@@ -617,7 +618,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
         if (more) load_stage(it + 1);
         process_stage(masked_tag, lds[it & 1], (q_first + it % n_qt) * QT);
         if (more) store_stage(lds[(it + 1) & 1], it + 1);
+        const unsigned now = WINDOW ? 0u : (unsigned)__builtin_amdgcn_s_memrealtime();
         __syncthreads();
+        if (!WINDOW) take_priority_turn(now, turn_class);  // the persistent grid only: see take_priority_turn
     };
 
     // Per query head of the group: the leading stages that touch this wavefront's causal diagonal (all stages if
