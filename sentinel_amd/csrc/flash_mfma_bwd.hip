@@ -17,6 +17,8 @@
 // In both kernels the score-like tiles are produced so that one lane owns one key (dK/dV kernel) or one
 // query (dQ kernel) and their registers are, after type conversion, directly the B operand of the
 // following product (see mfma_tile.h).
+// Without the sparse mask the grids are persistent (as many workgroups as the device runs at once, each walking the key
+// or query tiles of its XCD in snake order); result rows leave through LDS as whole rows (store_rows_via_lds).
 #include "flash_common.h"
 #include "mfma_tile.h"
 
