@@ -262,15 +262,28 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
         if (!WINDOW) take_priority_turn(now, turn_class);  // the persistent grid only: see take_priority_turn
     };
 
-    // Tiles that end at or before the first query of the workgroup need no mask for any wavefront; keep the count
-    // even so that the masked tail starts on LDS stage 0 again.
-    // Under the sparse mask a query tile sees few tiles and most of them cross a mask edge: all trips are masked ones.
-    const int bare_tiles = WINDOW ? 0 : (CAUSAL ? min(kv_tiles, qt * (kDqQueryTile / KT)) : T / KT) & ~1;
-    for (int j = 0; j < bare_tiles; j += 2) {
+    // Trips [bare_begin, bare_end) need no mask for any wavefront: their tiles end at or before the first query of the
+    // workgroup and, under the sparse mask, start inside the window of its last query (the trips before them hold the
+    // global tokens and the window's far edge, the ones after them the diagonal).  Both bounds are even so that every
+    // run of trips starts on LDS stage 0.
+    int bare_begin = 0;
+    int bare_end = (CAUSAL ? min(kv_tiles, qt * (kDqQueryTile / KT)) : T / KT) & ~1;
+    if (WINDOW) {
+        const int q_last = q_hi - 1;
+        const int inside = max(w_first, (max(0, q_last - g.window + 1) + KT - 1) / KT);  // first tile inside every window
+        bare_begin = (g_tiles + inside - w_first + 1) & ~1;
+        bare_end = (g_tiles + min(kv_tiles, qt * (kDqQueryTile / KT)) - w_first) & ~1;
+        if (bare_end <= bare_begin) bare_begin = bare_end = 0;
+        for (int j = 0; j < bare_begin; j += 2) {
+            tile_trip(std::true_type{}, j, k_lds0, v_lds0, k_lds1, v_lds1);
+            tile_trip(std::true_type{}, j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
+        }
+    }
+    for (int j = bare_begin; j < bare_end; j += 2) {
         tile_trip(std::false_type{}, j, k_lds0, v_lds0, k_lds1, v_lds1);
         tile_trip(std::false_type{}, j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
     }
-    for (int j = bare_tiles; j < n_trips; j += 2) {
+    for (int j = bare_end; j < n_trips; j += 2) {
         tile_trip(std::true_type{}, j, k_lds0, v_lds0, k_lds1, v_lds1);
         if (j + 1 < n_trips) tile_trip(std::true_type{}, j + 1, k_lds1, v_lds1, k_lds0, v_lds0);
     }
