@@ -36,7 +36,7 @@ SEEDS = {"c1": 1, "c2": 2, "c3": 3, "c4": 4, "c5": 5, "nstar": 6}
 KERNEL_UNITS = {"fwd_mfma": 2.0, "dkdv_mfma": 4.0, "dq_mfma": 1.0, "fwd_f32": 2.0, "dkdv_f32": 4.0, "dq_f32": 1.0}
 # HBM bytes per launch at the target shape, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/nstar_b4_h32_t4096_d128_bf16_counters.txt (scaled by a plain copy kernel of known size: x2.0 / x1.0)
-MEASURED_TRAFFIC_BYTES = {("nstar", "fwd_mfma"): 6.03e8, ("nstar", "dkdv_mfma"): 8.36e8, ("nstar", "dq_mfma"): 9.43e8}
+MEASURED_TRAFFIC_BYTES = {("nstar", "fwd_mfma"): 6.20e8, ("nstar", "dkdv_mfma"): 8.36e8, ("nstar", "dq_mfma"): 9.66e8}
 
 
 def make_inputs(torch, name):
