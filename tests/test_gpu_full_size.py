@@ -1,8 +1,11 @@
 """The baseline configurations at their full sizes (C ABI, [B,H,T,d]).
 
 The CPU oracle cannot run a whole configuration in seconds, so each case checks
-  * one (batch, K/V head) slice, with all query heads of its group, against the oracle at the full sequence
-    length (heads are independent, so the slice sees exactly the long-sequence tiling of the full launch);
+  * three (batch, K/V head) slices, each with all query heads of its group, against the oracle at the full sequence
+    length (heads are independent, so a slice sees exactly the long-sequence tiling of the full launch): the first
+    head of the first batch entry and the last head of the last one are the two ends of the persistent grids' walk
+    over the tiles, the third sits in the middle; every token's row is judged on its own (gpu_util.assert_close_lowp);
+  * the same for the column-layout call Sentinel makes (fp32 matrices, 16-bit arithmetic) at the two largest shapes;
   * properties that hold at any size and that an indexing or synchronisation mistake breaks:
     - scaling dO by 2 scales dQ, dK, dV by exactly 2 (bitwise in bf16: powers of two commute with every rounding);
     - causality: changing Q, K, V, dO behind position t leaves O, LSE and dQ before t bit-identical;
@@ -54,25 +57,65 @@ def _columns(x):
     return np.ascontiguousarray(x.float().cpu().numpy().transpose(0, 2, 1).reshape(h * d, t))
 
 
-@pytest.mark.parametrize("name", sorted(CONFIGS))
-def test_slice_matches_oracle_at_full_length(name):
+def _slice_of(where, b, hkv):
+    """(batch, K/V head) of the slice: the two ends of the persistent grids' walk over the tiles and the middle."""
+    return {"first": (0, 0), "middle": (b - 1, hkv // 2), "last": (b - 1, hkv - 1)}[where]
+
+
+def _check_slice(name, where, out, lse, dq, dk, dv, q, k, v, g):
     b, hq, hkv, t, d, dtype, _ = CONFIGS[name]
-    print(f"case {name} slice vs oracle", flush=True)
-    q, k, v, g = _inputs(name)
-    out, lse, dq, dk, dv = _run(q, k, v, g)
     group = hq // hkv
-    bi, kvh = b - 1, hkv // 2  # one (batch, K/V head) pair in the middle of the grid
+    bi, kvh = _slice_of(where, b, hkv)
     hs = slice(kvh * group, (kvh + 1) * group)
     want = gpu_util.oracle(_columns(q[bi, hs]), _columns(k[bi, kvh:kvh + 1]), _columns(v[bi, kvh:kvh + 1]),
                            _columns(g[bi, hs]), group, 1, d, t, 1)
-    gpu_util.assert_close_lowp(_columns(out[bi, hs]), want["out"], "out")
+    gpu_util.assert_close_lowp(_columns(out[bi, hs]), want["out"], "out", d)
     got_lse = lse[bi, hs].float().cpu().numpy()
     assert np.max(np.abs(got_lse - want["lse"][:, :t])) <= 2e-3, "lse"
-    gpu_util.assert_close_lowp(_columns(dq[bi, hs]), want["dq"], "dq")
-    gpu_util.assert_close_lowp(_columns(dk[bi, kvh:kvh + 1]), want["dk"], "dk")
-    gpu_util.assert_close_lowp(_columns(dv[bi, kvh:kvh + 1]), want["dv"], "dv")
+    gpu_util.assert_close_lowp(_columns(dq[bi, hs]), want["dq"], "dq", d)
+    gpu_util.assert_close_lowp(_columns(dk[bi, kvh:kvh + 1]), want["dk"], "dk", d)
+    gpu_util.assert_close_lowp(_columns(dv[bi, kvh:kvh + 1]), want["dv"], "dv", d)
+
+
+@pytest.mark.parametrize("where", ["first", "middle", "last"])
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_slice_matches_oracle_at_full_length(name, where):
+    print(f"case {name} {where} slice vs oracle", flush=True)
+    q, k, v, g = _inputs(name)
+    out, lse, dq, dk, dv = _run(q, k, v, g)
+    _check_slice(name, where, out, lse, dq, dk, dv, q, k, v, g)
     for x in (out, lse, dq, dk, dv):
         assert torch.isfinite(x.float()).all(), "non-finite value outside the checked slice"
+
+
+@pytest.mark.parametrize("where", ["first", "last"])
+@pytest.mark.parametrize("name", ["c4_gqa", "target_shape"])
+def test_drop_in_column_layout_at_full_length(name, where):
+    """The call Sentinel makes: fp32 [(head*d + dim), B*T] matrices through HipFlashAttention.forward_multi_head /
+    backward_multi_head with 16-bit arithmetic (layout conversion passes around the MFMA kernels), at the full size;
+    one (batch, K/V head) slice against the oracle."""
+    from sentinel_amd import HipFlashAttention
+    b, hq, hkv, t, d, dtype, _ = CONFIGS[name]
+    print(f"case {name} {where} column layout vs oracle", flush=True)
+    q, k, v, g = _inputs(name)  # 16-bit values, so the conversion pass rounds nothing on the way in
+
+    def columns(x):  # [B, H, T, d] -> fp32 [(h*d + c), b*T + t]
+        return x.float().permute(1, 3, 0, 2).reshape(x.shape[1] * d, b * t).contiguous()
+    qc, kc, vc, gc = (columns(x) for x in (q, k, v, g))
+    scale = 1.0 / np.sqrt(np.float32(d))
+    args = (hq, d, scale, True, 0, t, b)
+    kw = dict(kv_head_count=hkv, compute=dtype)
+    out, lse = HipFlashAttention.forward_multi_head(qc, kc, vc, None, None, *args, **kw)
+    dq, dk, dv = (torch.full_like(x, float("nan")) for x in (qc, kc, vc))
+    dq, dk, dv, _ = HipFlashAttention.backward_multi_head(qc, kc, vc, out, lse, gc, dq, dk, dv, None, *args, **kw)
+    torch.cuda.synchronize()
+
+    def bhtd(x, heads):  # back to [B, H, T, d]
+        return x.reshape(heads, d, b, t).permute(2, 0, 3, 1)
+    _check_slice(name, where, bhtd(out, hq), lse.reshape(hq, b, t).permute(1, 0, 2), bhtd(dq, hq), bhtd(dk, hkv),
+                 bhtd(dv, hkv), q, k, v, g)
+    for x in (out, lse, dq, dk, dv):
+        assert torch.isfinite(x).all(), "non-finite value outside the checked slice"
 
 
 @pytest.mark.parametrize("name", sorted(CONFIGS))

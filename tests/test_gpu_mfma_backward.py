@@ -34,7 +34,7 @@ def _run(dtype, shape, causal, sigma_qk=1.0, seed_extra=0):
     torch.cuda.synchronize()
     errs = {}
     for name, got, like in (("dq", dq, q), ("dk", dk, k), ("dv", dv, v)):
-        errs[name] = gpu_util.assert_close_lowp(gpu_util.bhtd_to_columns(got, like, 0), want[name], name)
+        errs[name] = gpu_util.assert_close_lowp(gpu_util.bhtd_to_columns(got, like, 0), want[name], name, d)
     return errs
 
 

@@ -71,7 +71,7 @@ def test_fused_rope_attention_matches_oracle(compute, shape):
         got = got.cpu().numpy()
         outside = np.isnan(want[key])
         assert np.all(got[outside] == sentinel), f"{key}: wrote outside the pack window"
-        gpu_util.assert_close_lowp(np.where(outside, np.nan, got), want[key], key)
+        gpu_util.assert_close_lowp(np.where(outside, np.nan, got), want[key], key, d)
     got = lse.cpu().numpy()
     outside = np.isnan(want["lse"])
     # the rotated Q, K are rounded to 16 bit before the scores are formed: LSE carries that rounding

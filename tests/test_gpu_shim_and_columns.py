@@ -58,7 +58,7 @@ def test_columns_layout_with_mfma_arithmetic(compute, shape):
         outside = np.isnan(want[key])
         assert np.all(got[outside] == sentinel), f"{key}: wrote outside the pack window"
         # the backward consumes `out` rounded to 16 bit a second time (fp32 -> 16 bit adapter), still within the bar
-        gpu_util.assert_close_lowp(np.where(outside, np.nan, got), want[key], key)
+        gpu_util.assert_close_lowp(np.where(outside, np.nan, got), want[key], key, d)
     got = lse.cpu().numpy()
     outside = np.isnan(want["lse"])
     assert np.all(got[outside] == sentinel)

@@ -103,11 +103,11 @@ def _bhtd(dtype, shape, seed_extra=0):
     dq, dk, dv = (torch.full_like(x, float("nan")) for x in (qd, kd, vd))
     flash_attention_backward(qd, kd, vd, out, lse, gd, dq=dq, dk=dk, dv=dv, **kw)
     torch.cuda.synchronize()
-    gpu_util.assert_close_lowp(gpu_util.bhtd_to_columns(out, q, 0), want["out"], "out")
+    gpu_util.assert_close_lowp(gpu_util.bhtd_to_columns(out, q, 0), want["out"], "out", d)
     got_lse = gpu_util.bht_to_columns(lse, hq, q.shape[1], 0)
     assert np.nanmax(np.abs(got_lse - want["lse"])) <= 2e-3, "lse"
     for name, got, like in (("dq", dq, q), ("dk", dk, k), ("dv", dv, v)):
-        gpu_util.assert_close_lowp(gpu_util.bhtd_to_columns(got, like, 0), want[name], name)
+        gpu_util.assert_close_lowp(gpu_util.bhtd_to_columns(got, like, 0), want[name], name, d)
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
@@ -138,7 +138,7 @@ def test_columns_with_mfma_arithmetic_and_fused_rotation():
     for key in ("out", "dq", "dk", "dv"):
         outside = np.isnan(want[key])
         assert np.all(got[key][outside] == sentinel), f"{key}: wrote outside the pack window"
-        gpu_util.assert_close_lowp(np.where(outside, np.nan, got[key]), want[key], key)
+        gpu_util.assert_close_lowp(np.where(outside, np.nan, got[key]), want[key], key, d)
 
 
 @pytest.mark.parametrize("dtype,d", [("bf16", 128), ("fp16", 64)])
