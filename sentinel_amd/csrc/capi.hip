@@ -94,6 +94,14 @@ int resolve(const char* op, int io_dtype, int compute_dtype, int layout, int q_h
     // every kernel indexes one tensor with 64-bit offsets but tiles with int
     if ((long long)pack_count * seq_len > 0x7fffffffLL / 4)
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s too many columns", op);
+    if (compute != SENTINEL_HIP_COMPUTE_F32) {
+        // the MFMA kernels address one head through a 32-bit buffer range and int byte offsets inside it
+        if ((long long)seq_len * head_dim * 2 > 0x7fffffffLL)
+            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s one head exceeds 2 GiB (seq_len * head_dim * 2 bytes)", op);
+        // the layout conversion launches one grid plane per (pack, head)
+        if (adapter && (long long)pack_count * q_heads > 65535)
+            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s more than 65535 (pack, head) pairs in the column layout", op);
+    }
 
     r->g = AttnGeom{q_heads, kv_heads, head_dim, seq_len, pack_count, scale, causal ? 1 : 0, 0, 0};
     r->io = io_dtype;
@@ -133,12 +141,17 @@ size_t workspace_need(const Resolved& r, bool backward) {
 extern "C" int sentinel_hip_flash_max_head_dim(void) { return 128; }
 
 extern "C" int sentinel_hip_device_available(void) {
-    int count = 0;
-    if (hipGetDeviceCount(&count) != hipSuccess) {
-        (void)hipGetLastError();
-        return 0;
-    }
-    return count > 0 ? 1 : 0;
+    // asked once per process: the answer cannot change under a running program, and a runtime query on every
+    // forward / backward call is host work on the launch path
+    static const int available = [] {
+        int count = 0;
+        if (hipGetDeviceCount(&count) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        return count > 0 ? 1 : 0;
+    }();
+    return available;
 }
 
 extern "C" const char* sentinel_hip_strerror(int code) {
@@ -188,6 +201,33 @@ int check_rope(const char* op, const float* cos_table, const float* sin_table, i
     return SENTINEL_HIP_OK;
 }
 
+// Rotary tables as handed in by the caller; validated against the RESOLVED sequence length (seq_len <= 0 means "the
+// rest of the window" in the column layout), never against the raw argument.
+struct RopeRequest {
+    const float* cos;
+    const float* sin;
+    int table_positions;
+    int position_offset;
+    bool requested;
+};
+const RopeRequest kNoRope = {nullptr, nullptr, 0, 0, false};
+
+int resolve_rope(const char* op, const RopeRequest& req, const Resolved& r, RopeTables* rope) {
+    *rope = RopeTables{nullptr, nullptr, 0};
+    if (!req.requested) return SENTINEL_HIP_OK;
+    const int rc = check_rope(op, req.cos, req.sin, req.table_positions, r.g.head_dim, req.position_offset, r.g.seq_len);
+    if (rc != SENTINEL_HIP_OK) return rc;
+    if (misaligned(req.cos) || misaligned(req.sin))
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
+    if (!r.adapter)
+        return fail(SENTINEL_HIP_UNSUPPORTED,
+                    "%s the rotation is fused into the layout conversion of fp32 column tensors with 16-bit arithmetic; "
+                    "rotate other tensors with sentinel_hip_rope_rotate",
+                    op);
+    *rope = RopeTables{req.cos, req.sin, req.position_offset};
+    return SENTINEL_HIP_OK;
+}
+
 // The layer's sparse mask (windowSize, globalTokenCount).  A window that covers the sequence is no window, and
 // without a window the global tokens change nothing: both collapse to the plain causal mask.
 struct SparseMask {
@@ -208,7 +248,7 @@ int apply_sparse_mask(const char* op, SparseMask mask, AttnGeom* g) {
 int flash_fwd(const char* op, const void* q, const void* k, const void* v, void* out, float* lse, int io_dtype,
               int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim, int stride_columns, int column_start,
               int seq_len, int pack_count, float scale, int causal, void* workspace, size_t workspace_bytes,
-              void* stream_ptr, RopeTables rope, SparseMask mask = kNoSparseMask) {
+              void* stream_ptr, const RopeRequest& rope_request, SparseMask mask = kNoSparseMask) {
     if (!q || !k || !v || !out || !lse) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
     Resolved r;
     const int rc = resolve(op, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns, column_start,
@@ -216,11 +256,9 @@ int flash_fwd(const char* op, const void* q, const void* k, const void* v, void*
     if (rc != SENTINEL_HIP_OK) return rc;
     const int mask_rc = apply_sparse_mask(op, mask, &r.g);
     if (mask_rc != SENTINEL_HIP_OK) return mask_rc;
-    if (rope.cos && !r.adapter)
-        return fail(SENTINEL_HIP_UNSUPPORTED,
-                    "%s the rotation is fused into the layout conversion of fp32 column tensors with 16-bit arithmetic; "
-                    "rotate other tensors with sentinel_hip_rope_rotate",
-                    op);
+    RopeTables rope;
+    const int rope_rc = resolve_rope(op, rope_request, r, &rope);
+    if (rope_rc != SENTINEL_HIP_OK) return rope_rc;
     if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
     hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
     const AttnGeom& g = r.g;
@@ -275,8 +313,8 @@ int flash_fwd(const char* op, const void* q, const void* k, const void* v, void*
 int flash_bwd(const char* op, const void* q, const void* k, const void* v, const void* out, const float* lse,
               const void* d_out, void* dq, void* dk, void* dv, float* delta, int io_dtype, int compute_dtype, int layout,
               int q_heads, int kv_heads, int head_dim, int stride_columns, int column_start, int seq_len, int pack_count,
-              float scale, int causal, void* workspace, size_t workspace_bytes, void* stream_ptr, RopeTables rope,
-              SparseMask mask = kNoSparseMask) {
+              float scale, int causal, void* workspace, size_t workspace_bytes, void* stream_ptr,
+              const RopeRequest& rope_request, SparseMask mask = kNoSparseMask) {
     if (!q || !k || !v || !out || !lse || !d_out || !dq || !dk || !dv || !delta)
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
     Resolved r;
@@ -285,11 +323,9 @@ int flash_bwd(const char* op, const void* q, const void* k, const void* v, const
     if (rc != SENTINEL_HIP_OK) return rc;
     const int mask_rc = apply_sparse_mask(op, mask, &r.g);
     if (mask_rc != SENTINEL_HIP_OK) return mask_rc;
-    if (rope.cos && !r.adapter)
-        return fail(SENTINEL_HIP_UNSUPPORTED,
-                    "%s the rotation is fused into the layout conversion of fp32 column tensors with 16-bit arithmetic; "
-                    "rotate other tensors with sentinel_hip_rope_rotate",
-                    op);
+    RopeTables rope;
+    const int rope_rc = resolve_rope(op, rope_request, r, &rope);
+    if (rope_rc != SENTINEL_HIP_OK) return rope_rc;
     if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
     hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
     const AttnGeom& g = r.g;
@@ -369,10 +405,9 @@ extern "C" int sentinel_hip_flash_fwd(const void* q, const void* k, const void* 
                                       int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
                                       int stride_columns, int column_start, int seq_len, int pack_count, float scale,
                                       int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
-    const RopeTables none = {nullptr, nullptr, 0};
     return flash_fwd("sentinel_hip_flash_fwd", q, k, v, out, lse, io_dtype, compute_dtype, layout, q_heads, kv_heads,
                      head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes,
-                     stream_ptr, none);
+                     stream_ptr, kNoRope);
 }
 
 extern "C" int sentinel_hip_flash_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
@@ -380,10 +415,9 @@ extern "C" int sentinel_hip_flash_bwd(const void* q, const void* k, const void* 
                                       int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
                                       int stride_columns, int column_start, int seq_len, int pack_count, float scale,
                                       int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
-    const RopeTables none = {nullptr, nullptr, 0};
     return flash_bwd("sentinel_hip_flash_bwd", q, k, v, out, lse, d_out, dq, dk, dv, delta, io_dtype, compute_dtype, layout,
                      q_heads, kv_heads, head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal,
-                     workspace, workspace_bytes, stream_ptr, none);
+                     workspace, workspace_bytes, stream_ptr, kNoRope);
 }
 
 extern "C" int sentinel_hip_flash_fwd_rope(const void* q, const void* k, const void* v, void* out, float* lse,
@@ -392,14 +426,10 @@ extern "C" int sentinel_hip_flash_fwd_rope(const void* q, const void* k, const v
                                            int kv_heads, int head_dim, int stride_columns, int column_start, int seq_len,
                                            int pack_count, float scale, int causal, void* workspace,
                                            size_t workspace_bytes, void* stream_ptr) {
-    const char* op = "sentinel_hip_flash_fwd_rope";
-    const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
-    if (rc != SENTINEL_HIP_OK) return rc;
-    if (misaligned(cos_table) || misaligned(sin_table))
-        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
-    const RopeTables rope = {cos_table, sin_table, position_offset};
-    return flash_fwd(op, q, k, v, out, lse, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns,
-                     column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes, stream_ptr, rope);
+    const RopeRequest rope = {cos_table, sin_table, table_positions, position_offset, true};
+    return flash_fwd("sentinel_hip_flash_fwd_rope", q, k, v, out, lse, io_dtype, compute_dtype, layout, q_heads, kv_heads,
+                     head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes,
+                     stream_ptr, rope);
 }
 
 extern "C" int sentinel_hip_flash_bwd_rope(const void* q, const void* k, const void* v, const void* out, const float* lse,
@@ -409,15 +439,10 @@ extern "C" int sentinel_hip_flash_bwd_rope(const void* q, const void* k, const v
                                            int kv_heads, int head_dim, int stride_columns, int column_start, int seq_len,
                                            int pack_count, float scale, int causal, void* workspace,
                                            size_t workspace_bytes, void* stream_ptr) {
-    const char* op = "sentinel_hip_flash_bwd_rope";
-    const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
-    if (rc != SENTINEL_HIP_OK) return rc;
-    if (misaligned(cos_table) || misaligned(sin_table))
-        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
-    const RopeTables rope = {cos_table, sin_table, position_offset};
-    return flash_bwd(op, q, k, v, out, lse, d_out, dq, dk, dv, delta, io_dtype, compute_dtype, layout, q_heads, kv_heads,
-                     head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes,
-                     stream_ptr, rope);
+    const RopeRequest rope = {cos_table, sin_table, table_positions, position_offset, true};
+    return flash_bwd("sentinel_hip_flash_bwd_rope", q, k, v, out, lse, d_out, dq, dk, dv, delta, io_dtype, compute_dtype,
+                     layout, q_heads, kv_heads, head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal,
+                     workspace, workspace_bytes, stream_ptr, rope);
 }
 
 extern "C" int sentinel_hip_flash_fwd_sparse(const void* q, const void* k, const void* v, void* out, float* lse,
@@ -426,18 +451,11 @@ extern "C" int sentinel_hip_flash_fwd_sparse(const void* q, const void* k, const
                                              int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
                                              int stride_columns, int column_start, int seq_len, int pack_count, float scale,
                                              int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
-    const char* op = "sentinel_hip_flash_fwd_sparse";
-    RopeTables rope = {nullptr, nullptr, 0};
-    if (cos_table || sin_table) {
-        const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
-        if (rc != SENTINEL_HIP_OK) return rc;
-        if (misaligned(cos_table) || misaligned(sin_table))
-            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
-        rope = RopeTables{cos_table, sin_table, position_offset};
-    }
-    return flash_fwd(op, q, k, v, out, lse, io_dtype, compute_dtype, layout, q_heads, kv_heads, head_dim, stride_columns,
-                     column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes, stream_ptr, rope,
-                     SparseMask{window_size, global_token_count});
+    // both tables NULL: no rotation; one without the other is reported as "empty tables"
+    const RopeRequest rope = {cos_table, sin_table, table_positions, position_offset, cos_table || sin_table};
+    return flash_fwd("sentinel_hip_flash_fwd_sparse", q, k, v, out, lse, io_dtype, compute_dtype, layout, q_heads, kv_heads,
+                     head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes,
+                     stream_ptr, rope, SparseMask{window_size, global_token_count});
 }
 
 extern "C" int sentinel_hip_flash_bwd_sparse(const void* q, const void* k, const void* v, const void* out, const float* lse,
@@ -447,18 +465,10 @@ extern "C" int sentinel_hip_flash_bwd_sparse(const void* q, const void* k, const
                                              int compute_dtype, int layout, int q_heads, int kv_heads, int head_dim,
                                              int stride_columns, int column_start, int seq_len, int pack_count, float scale,
                                              int causal, void* workspace, size_t workspace_bytes, void* stream_ptr) {
-    const char* op = "sentinel_hip_flash_bwd_sparse";
-    RopeTables rope = {nullptr, nullptr, 0};
-    if (cos_table || sin_table) {
-        const int rc = check_rope(op, cos_table, sin_table, table_positions, head_dim, position_offset, seq_len);
-        if (rc != SENTINEL_HIP_OK) return rc;
-        if (misaligned(cos_table) || misaligned(sin_table))
-            return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
-        rope = RopeTables{cos_table, sin_table, position_offset};
-    }
-    return flash_bwd(op, q, k, v, out, lse, d_out, dq, dk, dv, delta, io_dtype, compute_dtype, layout, q_heads, kv_heads,
-                     head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal, workspace, workspace_bytes,
-                     stream_ptr, rope, SparseMask{window_size, global_token_count});
+    const RopeRequest rope = {cos_table, sin_table, table_positions, position_offset, cos_table || sin_table};
+    return flash_bwd("sentinel_hip_flash_bwd_sparse", q, k, v, out, lse, d_out, dq, dk, dv, delta, io_dtype, compute_dtype,
+                     layout, q_heads, kv_heads, head_dim, stride_columns, column_start, seq_len, pack_count, scale, causal,
+                     workspace, workspace_bytes, stream_ptr, rope, SparseMask{window_size, global_token_count});
 }
 
 extern "C" int sentinel_hip_rope_rotate(float* tensor, int heads, int head_dim, int stride_columns, int column_start,
@@ -476,6 +486,8 @@ extern "C" int sentinel_hip_rope_rotate(float* tensor, int heads, int head_dim, 
                               segment_length > 0 ? segment_length : columns);
     if (rc != SENTINEL_HIP_OK) return rc;
     if (position_offset < 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s negative positionOffset", op);
+    if ((long long)heads * (head_dim / 2) > 65535)  // one grid row per (head, pair)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s more than 65535 (head, pair) rows", op);
     if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
     const hipError_t err = launch_rope_rotate_f32(tensor + column_start, heads, head_dim, stride_columns, columns,
                                                   position_offset, segment_length, cos_table, sin_table, inverse != 0,

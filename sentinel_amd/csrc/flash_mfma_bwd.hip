@@ -74,9 +74,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     // K / V through one L2); round r hands the XCD's tiles [r S, (r + 1) S) to its S workgroups, forwards in even
     // rounds and backwards in odd ones, so long and short tiles alternate.
     const unsigned turn_class = priority_turn_class();
-    const int xcd = (int)blockIdx.x % 8;
-    const int slot = (int)blockIdx.x / 8;
-    const int slots = (int)gridDim.x / 8;
+    const int xcd = (int)blockIdx.x % kXcds;
+    const int slot = (int)blockIdx.x / kXcds;
+    const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
     const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
     const int tile_id = xcd * tiles_per_xcd + local_tile;
@@ -295,19 +295,6 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     }  // next tile of this workgroup (the last trip ended with a barrier: the LDS stages are free)
 }
 
-// Workgroups the device runs at once, per XCD (8 XCDs): occupancy of the kernel times the compute units of an XCD.
-template <typename Kernel>
-int resident_workgroups_per_xcd(Kernel kernel, int threads, size_t dynamic_lds) {
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess || per_cu <= 0) per_cu = 1;
-    int device = 0;
-    int cus = 0;
-    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
-        cus <= 0)
-        cus = 256;
-    return per_cu * ((cus + 7) / 8);
-}
-
 constexpr int kDkvKeyTile = 128;
 constexpr int kDkvQueryTile = 64;
 
@@ -411,8 +398,8 @@ __device__ __forceinline__ int dkv_query_tiles(const AttnGeom& g, int k0, int q_
 __device__ __forceinline__ bool dkv_tile_of_workgroup(int xcd, int local, int per_xcd, int k_tiles, int total_tiles,
                                                       int front_tiles, int& bkv, int& ktile) {
     const int heads = total_tiles / k_tiles;
-    if (front_tiles > 0 && heads % 8 == 0) {
-        const int heads_per_xcd = heads / 8;
+    if (front_tiles > 0 && heads % kXcds == 0) {
+        const int heads_per_xcd = heads / kXcds;
         const int front = front_tiles * heads_per_xcd;
         if (local < front) {
             ktile = local / heads_per_xcd;
@@ -458,9 +445,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     // persistent workgroups walking the XCD's key tiles in snake order (see dq_mfma_kernel)
     const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
     const unsigned turn_class = priority_turn_class();
-    const int xcd = (int)blockIdx.x % 8;
-    const int slot = (int)blockIdx.x / 8;
-    const int slots = (int)gridDim.x / 8;
+    const int xcd = (int)blockIdx.x % kXcds;
+    const int slot = (int)blockIdx.x / kXcds;
+    const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
     const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
     int bkv, ktile;
@@ -695,9 +682,9 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
 
     // persistent workgroups walking the XCD's key tiles in snake order (see dq_mfma_kernel)
     const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
-    const int xcd = (int)blockIdx.x % 8;
-    const int slot = (int)blockIdx.x / 8;
-    const int slots = (int)gridDim.x / 8;
+    const int xcd = (int)blockIdx.x % kXcds;
+    const int slot = (int)blockIdx.x / kXcds;
+    const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
     const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
     int bkv, ktile;
@@ -1007,12 +994,12 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
     {
         const int q_tiles = (T + kDqQueryTile - 1) / kDqQueryTile;
         const int total = g.packs * g.q_heads * q_tiles;
-        const int tiles_per_xcd = (total + 7) / 8;
+        const int tiles_per_xcd = (total + kXcds - 1) / kXcds;
         auto launch = [&](auto kernel) {
             static const int resident = resident_workgroups_per_xcd(kernel, kBwdThreads, 0);  // per kernel instantiation
             // under the sparse mask tile lengths no longer grow with the tile index, and one workgroup per tile handed out
             // as slots free up is 6 - 13 % faster than the fixed snake assignment
-            const int grid = 8 * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            const int grid = kXcds * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
             KernelTimer timer("dq_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp, lse, delta, dqp, lm, g,
                                q_tiles, total, tiles_per_xcd);
@@ -1029,14 +1016,14 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
     // dK, dV
     const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
     const int total = g.packs * g.kv_heads * k_tiles;
-    const int tiles_per_xcd = (total + 7) / 8;
+    const int tiles_per_xcd = (total + kXcds - 1) / kXcds;
     if constexpr (D <= 64) {
         const size_t smem = 2 * sizeof(DkvLds<D>);
         auto launch = [&](auto kernel) {
             static const int resident = resident_workgroups_per_xcd(kernel, kBwdThreads, smem);  // per kernel instantiation
             // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
             // dispatched in order (long ones first), balances better than a fixed assignment
-            const int grid = 8 * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            const int grid = kXcds * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp, dvp, lm, g,
                                k_tiles, total, tiles_per_xcd);
@@ -1058,7 +1045,7 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
             static const int resident = resident_workgroups_per_xcd(kernel, kDkvSplitThreads, smem);
             // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
             // dispatched in order (long ones first), balances better than a fixed assignment
-            const int grid = 8 * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            const int grid = kXcds * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp, dvp, lm, g,
                                k_tiles, total, tiles_per_xcd);

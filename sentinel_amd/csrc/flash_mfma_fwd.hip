@@ -68,9 +68,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     // L2.  Round r hands the XCD's tiles [r S, (r + 1) S) to its S workgroups, forwards in even rounds and backwards
     // in odd ones: long and short tiles alternate and every workgroup ends up with about the same work.
     const unsigned turn_class = priority_turn_class();
-    const int xcd = (int)blockIdx.x % 8;
-    const int slot = (int)blockIdx.x / 8;
-    const int slots = (int)gridDim.x / 8;
+    const int xcd = (int)blockIdx.x % kXcds;
+    const int slot = (int)blockIdx.x / kXcds;
+    const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
     const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
     const int tile_id = xcd * tiles_per_xcd + local_tile;
@@ -278,25 +278,12 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     }  // next tile of this workgroup (the last trip ended with a barrier: the LDS stages are free)
 }
 
-// Workgroups the device runs at once, per XCD (8 XCDs): occupancy of the kernel times the compute units of an XCD.
-template <typename Kernel>
-int resident_workgroups_per_xcd(Kernel kernel, int threads, size_t dynamic_lds) {
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess || per_cu <= 0) per_cu = 1;
-    int device = 0;
-    int cus = 0;
-    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
-        cus <= 0)
-        cus = 256;
-    return per_cu * ((cus + 7) / 8);
-}
-
 template <typename E, int D>
 hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm, AttnGeom g,
                    hipStream_t stream) {
     const int q_tiles = (g.seq_len + kFwdQueryTile - 1) / kFwdQueryTile;
     const int total = g.packs * g.q_heads * q_tiles;
-    const int tiles_per_xcd = (total + 7) / 8;
+    const int tiles_per_xcd = (total + kXcds - 1) / kXcds;
     auto qp = static_cast<const unsigned short*>(q);
     auto kp = static_cast<const unsigned short*>(k);
     auto vp = static_cast<const unsigned short*>(v);
@@ -305,7 +292,7 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
         static const int resident = resident_workgroups_per_xcd(kernel, kFwdThreads, 0);  // per kernel instantiation
         // under the sparse mask tile lengths no longer grow with the tile index, and one workgroup per tile handed out
         // as slots free up is 6 - 13 % faster than the fixed snake assignment
-        const int grid = 8 * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+        const int grid = kXcds * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
         KernelTimer timer("fwd_mfma", stream);
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm, g, q_tiles, total,
                            tiles_per_xcd);

@@ -4,6 +4,7 @@
 // made with timing on must not be captured into a graph.
 #include "flash_common.h"
 
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -18,7 +19,7 @@ struct Record {
 };
 
 std::mutex g_mutex;
-bool g_enabled = false;
+std::atomic<bool> g_enabled{false};  // read without the lock on every launch
 std::vector<Record> g_records;
 std::vector<hipEvent_t> g_pool;
 
@@ -36,8 +37,8 @@ hipEvent_t take_event() {
 }  // namespace
 
 KernelTimer::KernelTimer(const char* name, hipStream_t stream) : name_(name), stream_(stream), start_(nullptr) {
+    if (!g_enabled.load(std::memory_order_relaxed)) return;  // timing off: no lock, no host state touched
     std::lock_guard<std::mutex> lock(g_mutex);
-    if (!g_enabled) return;
     start_ = take_event();
     if (start_) (void)hipEventRecord(start_, stream_);
 }
@@ -56,8 +57,8 @@ KernelTimer::~KernelTimer() {
 
 int timing_set_enabled(int enabled) {
     std::lock_guard<std::mutex> lock(g_mutex);
-    const int before = g_enabled ? 1 : 0;
-    g_enabled = enabled != 0;
+    const int before = g_enabled.load() ? 1 : 0;
+    g_enabled.store(enabled != 0);
     return before;
 }
 

@@ -298,5 +298,22 @@ __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], 
     }
 }
 
+// The device is built from kXcds accelerator dies (XCDs), each with its own L2; the hardware deals workgroup ids
+// round-robin to them, so workgroup id % kXcds names the die a workgroup runs on.
+constexpr int kXcds = 8;
+
+// Workgroups the device runs at once, per XCD: occupancy of the kernel times the compute units of an XCD.
+template <typename Kernel>
+inline int resident_workgroups_per_xcd(Kernel kernel, int threads, size_t dynamic_lds) {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess || per_cu <= 0) per_cu = 1;
+    int device = 0;
+    int cus = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+        cus <= 0)
+        cus = 256;
+    return per_cu * ((cus + kXcds - 1) / kXcds);
+}
+
 }  // namespace sentinel_hip
 #endif

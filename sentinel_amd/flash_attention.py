@@ -117,19 +117,49 @@ def _ptr(t):
 
 
 def _ensure_size(t, rows, cols, like):
-    """CudaMatrix::ensureSize for an optional output tensor."""
+    """CudaMatrix::ensureSize for an optional output tensor: a tensor of another shape is replaced, one of the right
+    shape must be a contiguous fp32 matrix on the inputs' device (its raw pointer crosses the C ABI)."""
     if t is None or tuple(t.shape) != (rows, cols):
         return torch.empty((rows, cols), dtype=torch.float32, device=like.device)
+    _require(t, (rows, cols), torch.float32, like.device, "output matrix")
     return t
+
+
+def _require(t, shape, dtype, device, what):
+    """Every tensor whose pointer is handed to the library is checked here: the C ABI sees addresses only."""
+    if not isinstance(t, torch.Tensor):
+        raise ValueError(f"{what}: expected a tensor")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{what}: shape {tuple(t.shape)} where {tuple(shape)} is expected")
+    if t.dtype != dtype:
+        raise ValueError(f"{what}: dtype {t.dtype} where {dtype} is expected")
+    if not t.is_contiguous():
+        raise ValueError(f"{what}: must be contiguous")
+    if t.device != device:
+        raise ValueError(f"{what}: on {t.device}, the inputs are on {device}")
+
+
+def _on_stream(stream, *temporaries):
+    """Temporaries come from torch's caching allocator, which hands a freed block to later work on the CURRENT stream;
+    when the kernels run on another stream, tell the allocator so."""
+    if stream is None:
+        return
+    for t in temporaries:
+        if t is not None and stream != torch.cuda.current_stream(t.device):
+            t.record_stream(stream)
 
 
 def _workspace(lib, io, compute, layout, hq, hkv, d, t, packs, backward, device, workspace):
     need = lib.sentinel_hip_flash_workspace_bytes(io, compute, layout, hq, hkv, d, t, packs, int(backward))
     if need == 0:
-        return None, 0
-    if workspace is None or workspace.numel() * workspace.element_size() < need:
-        workspace = torch.empty(need, dtype=torch.uint8, device=device)
-    return workspace, need
+        return None, 0, None
+    if workspace is not None:
+        if not workspace.is_contiguous() or workspace.device != device:
+            raise ValueError("workspace must be a contiguous tensor on the inputs' device")
+        if workspace.numel() * workspace.element_size() >= need:
+            return workspace, workspace.numel() * workspace.element_size(), None
+    own = torch.empty(need, dtype=torch.uint8, device=device)
+    return own, need, own
 
 
 def _rope_args(rope, head_dimension):
@@ -202,8 +232,9 @@ class HipFlashAttention:
         log_sum_exp = _ensure_size(log_sum_exp, head_count, cols, query)
         comp = _COMPUTE_CODE[compute]
         seq = column_count if column_count > 0 else cols - column_start
-        ws, ws_bytes = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1),
-                                  max(pack_count, 1), False, query.device, workspace)
+        ws, ws_bytes, ws_own = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1),
+                                          max(pack_count, 1), False, query.device, workspace)
+        _on_stream(stream, ws_own)
         tail = (F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start, column_count,
                 pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes, _stream_handle(stream))
         if window_size > 0 or global_token_count != 0:
@@ -244,6 +275,8 @@ class HipFlashAttention:
             raise ValueError("HipFlashAttention::backwardMultiHead outGradient shape mismatch")
         if tuple(log_sum_exp.shape) != (head_count, cols):
             raise ValueError("HipFlashAttention::backwardMultiHead logSumExp shape mismatch")
+        for t, what in ((out, "out"), (out_gradient, "outGradient"), (log_sum_exp, "logSumExp")):
+            _require(t, None, torch.float32, query.device, "HipFlashAttention::backwardMultiHead " + what)
         seq = column_count if column_count > 0 else cols - column_start
         packs = max(pack_count, 1)
         query_gradient = _ensure_size(query_gradient, rows, cols, query)
@@ -251,8 +284,9 @@ class HipFlashAttention:
         value_gradient = _ensure_size(value_gradient, value.shape[0], cols, query)
         delta_workspace = _ensure_size(delta_workspace, head_count, packs * max(seq, 1), query)
         comp = _COMPUTE_CODE[compute]
-        ws, ws_bytes = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1), packs,
-                                  True, query.device, workspace)
+        ws, ws_bytes, ws_own = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1),
+                                          packs, True, query.device, workspace)
+        _on_stream(stream, ws_own)
         head = (_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp), _ptr(out_gradient), _ptr(query_gradient),
                 _ptr(key_gradient), _ptr(value_gradient), _ptr(delta_workspace))
         tail = (F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start, column_count,
@@ -322,11 +356,15 @@ def decode_attention(query, key_cache, value_cache, length, head_count, head_dim
     scale = 1.0 / math.sqrt(head_dimension) if scale is None else float(scale)
     out = _ensure_size(out, head_count * head_dimension, 1, query)
     need = lib.sentinel_hip_decode_workspace_bytes(head_count, head_dimension, max(int(length), 1))
+    if workspace is not None and (not workspace.is_contiguous() or workspace.device != query.device):
+        raise ValueError("decode_attention workspace must be a contiguous tensor on the inputs' device")
     if workspace is None or workspace.numel() * workspace.element_size() < need:
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=query.device)
+        _on_stream(stream, workspace)
     _check(lib.sentinel_hip_decode_attention(_ptr(query), _ptr(key_cache), _ptr(value_cache), _ptr(out), head_count, kv_heads,
                                              head_dimension, int(key_cache.shape[1]), int(length), scale, int(window_size),
-                                             int(global_token_count), _ptr(workspace), need, _stream_handle(stream)))
+                                             int(global_token_count), _ptr(workspace),
+                                             workspace.numel() * workspace.element_size(), _stream_handle(stream)))
     return out
 
 
@@ -352,6 +390,8 @@ def flash_attention_forward(q, k, v, scale=None, causal=True, out=None, lse=None
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     out = torch.empty_like(q) if out is None else out
     lse = torch.empty((b, hq, t), dtype=torch.float32, device=q.device) if lse is None else lse
+    _require(out, q.shape, q.dtype, q.device, "flash_attention_forward out")
+    _require(lse, (b, hq, t), torch.float32, q.device, "flash_attention_forward lse")
     code = _DTYPE_CODE[q.dtype]
     if window_size > 0 or global_token_count != 0:
         _check(lib.sentinel_hip_flash_fwd_sparse(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), None, None, 0, 0,
@@ -373,7 +413,16 @@ def flash_attention_backward(q, k, v, out, lse, d_out, scale=None, causal=True, 
     dq = torch.empty_like(q) if dq is None else dq
     dk = torch.empty_like(k) if dk is None else dk
     dv = torch.empty_like(v) if dv is None else dv
-    delta = torch.empty((hq, b * t), dtype=torch.float32, device=q.device) if delta is None else delta
+    own_delta = delta is None
+    delta = torch.empty((hq, b * t), dtype=torch.float32, device=q.device) if own_delta else delta
+    for x, like, what in ((out, q, "out"), (d_out, q, "d_out"), (dq, q, "dq"), (dk, k, "dk"), (dv, v, "dv")):
+        _require(x, like.shape, q.dtype, q.device, "flash_attention_backward " + what)
+    _require(lse, (b, hq, t), torch.float32, q.device, "flash_attention_backward lse")
+    _require(delta, None, torch.float32, q.device, "flash_attention_backward delta")
+    if delta.numel() < hq * b * t:
+        raise ValueError(f"flash_attention_backward delta: {delta.numel()} floats where {hq * b * t} are needed")
+    if own_delta:
+        _on_stream(stream, delta)
     code = _DTYPE_CODE[q.dtype]
     head = (_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(delta))
     tail = (code, COMPUTE_AUTO, LAYOUT_BHTD, hq, hkv, d, 0, 0, t, b, scale, int(bool(causal)), None, 0, _stream_handle(stream))

@@ -76,6 +76,27 @@ def test_sparse_rope_and_decode_validation_without_a_gpu(lib):
         assert call() == 3 and b"no HIP device" in lib.sentinel_hip_last_error()
         assert call(window=0, causal=0) == 3  # no window: the causal flag is free again
 
+    # seq_len <= 0 means "the rest of the window" in the column layout: the tables are checked against the resolved
+    # length (here 256 columns against 4 table rows), not against the raw argument
+    rope_fwd = lib.sentinel_hip_flash_fwd_rope
+    ws = ctypes.c_void_p(256)
+    for seq_len in (256, 0):
+        assert rope_fwd(one, one, one, one, one, one, one, 4, 0, 0, 1, 0, 2, 2, 64, 256, 0, seq_len, 1, 0.125, 1, ws, 1 << 30,
+                        None) == 1, seq_len
+        assert b"position exceeds RoPE table" in lib.sentinel_hip_last_error()
+    rope_bwd = lib.sentinel_hip_flash_bwd_rope
+    assert rope_bwd(one, one, one, one, one, one, one, one, one, one, one, one, 4, 0, 0, 1, 0, 2, 2, 64, 256, 0, 0, 1, 0.125,
+                    1, ws, 1 << 30, None) == 1
+    assert b"position exceeds RoPE table" in lib.sentinel_hip_last_error()
+    assert sparse(one, one, one, one, one, one, one, 4, 0, 8, 0, 0, 1, 0, 2, 2, 64, 256, 0, 0, 1, 0.125, 1, ws, 1 << 30,
+                  None) == 1 and b"position exceeds RoPE table" in lib.sentinel_hip_last_error()
+    # limits of the 32-bit addressing inside one head and of the conversion grid
+    fwd = lib.sentinel_hip_flash_fwd
+    assert fwd(one, one, one, one, one, 1, -1, 1, 1, 1, 128, 0, 0, 1 << 24, 1, 0.1, 1, None, 0, None) == 1
+    assert b"exceeds 2 GiB" in lib.sentinel_hip_last_error()
+    assert fwd(one, one, one, one, one, 0, 1, 0, 70000, 70000, 64, 8, 0, 8, 1, 0.1, 1, ws, 1 << 40, None) == 1
+    assert b"65535" in lib.sentinel_hip_last_error()
+
     rotate = lib.sentinel_hip_rope_rotate
     assert rotate(one, 2, 15, 12, 0, 12, 0, 0, one, one, 32, 0, None) == 1 and b"invalid rope dims" in lib.sentinel_hip_last_error()
     assert rotate(one, 2, 16, 12, 0, 12, 0, 0, one, one, 10, 0, None) == 1 and b"position exceeds RoPE table" in lib.sentinel_hip_last_error()
