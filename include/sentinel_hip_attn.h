@@ -184,6 +184,21 @@ SENTINEL_HIP_API int sentinel_hip_decode_attention(const float* query, const flo
                                   int window_size, int global_token_count, void* workspace, size_t workspace_bytes,
                                   void* stream);
 
+/*
+ * sentinel_hip_decode_attention without a workspace argument and without any allocation. It has no counterpart in
+ * the reference; it is for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc. The partial results live in a device array that is part of the library
+ * (SENTINEL_HIP_DECODE_STATIC_SCRATCH_BYTES per GPU, held until the process ends); a call whose
+ * sentinel_hip_decode_workspace_bytes(q_heads, head_dim, length) exceeds it returns SENTINEL_HIP_INVALID_ARGUMENT.
+ * Arguments, results and kernels are those of sentinel_hip_decode_attention. All calls on one GPU share that GPU's
+ * array: calls that overlap in time on one GPU (different streams, threads) race; calls on one stream do not. The
+ * first call on a device looks the array's address up (no allocation, no synchronisation); make it before capture.
+ */
+#define SENTINEL_HIP_DECODE_STATIC_SCRATCH_BYTES ((size_t)4 << 20)
+SENTINEL_HIP_API int sentinel_hip_decode_attention_static(const float* query, const float* key_cache, const float* value_cache,
+                                         float* out, int q_heads, int kv_heads, int head_dim, int cache_stride, int length,
+                                         float scale, int window_size, int global_token_count, void* stream);
+
 /* Largest head_dim any kernel here accepts (the CUDA path's CudaFlashAttention::maxHeadDimension is 64). */
 SENTINEL_HIP_API int sentinel_hip_flash_max_head_dim(void);
 

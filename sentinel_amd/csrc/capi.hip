@@ -501,11 +501,11 @@ extern "C" size_t sentinel_hip_decode_workspace_bytes(int q_heads, int head_dim,
     return align_up(decode_workspace_bytes(q_heads, head_dim, length));
 }
 
-extern "C" int sentinel_hip_decode_attention(const float* query, const float* key_cache, const float* value_cache, float* out,
-                                             int q_heads, int kv_heads, int head_dim, int cache_stride, int length,
-                                             float scale, int window_size, int global_token_count, void* workspace,
-                                             size_t workspace_bytes, void* stream_ptr) {
-    const char* op = "sentinel_hip_decode_attention";
+namespace {
+
+// argument checks shared by the two decode entry points (everything but the workspace)
+int check_decode(const char* op, const float* query, const float* key_cache, const float* value_cache, const float* out,
+                 int q_heads, int kv_heads, int head_dim, int cache_stride, int length, float scale, int global_token_count) {
     if (!query || !key_cache || !value_cache || !out) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty input", op);
     if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s invalid head geometry", op);
     if (q_heads % kv_heads != 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s headCount must be divisible by kvHeadCount", op);
@@ -518,6 +518,19 @@ extern "C" int sentinel_hip_decode_attention(const float* query, const float* ke
     if (group != 1 && group != 2 && group != 4 && group != 8)
         return fail(SENTINEL_HIP_UNSUPPORTED, "%s query heads per K/V head must be 1, 2, 4 or 8 (got %d)", op, group);
     if (head_dim % 8 != 0) return fail(SENTINEL_HIP_UNSUPPORTED, "%s head_dim must be a multiple of 8", op);
+    return SENTINEL_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" int sentinel_hip_decode_attention(const float* query, const float* key_cache, const float* value_cache, float* out,
+                                             int q_heads, int kv_heads, int head_dim, int cache_stride, int length,
+                                             float scale, int window_size, int global_token_count, void* workspace,
+                                             size_t workspace_bytes, void* stream_ptr) {
+    const char* op = "sentinel_hip_decode_attention";
+    const int rc = check_decode(op, query, key_cache, value_cache, out, q_heads, kv_heads, head_dim, cache_stride, length, scale,
+                                global_token_count);
+    if (rc != SENTINEL_HIP_OK) return rc;
     const size_t need = sentinel_hip_decode_workspace_bytes(q_heads, head_dim, length);
     if (!workspace || workspace_bytes < need || misaligned(workspace))
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s needs %zu bytes of 16-byte aligned workspace", op, need);
@@ -525,6 +538,31 @@ extern "C" int sentinel_hip_decode_attention(const float* query, const float* ke
     const hipError_t err = launch_decode_attention(query, key_cache, value_cache, out, q_heads, kv_heads, head_dim,
                                                    cache_stride, length, scale, window_size, global_token_count,
                                                    static_cast<float*>(workspace), static_cast<hipStream_t>(stream_ptr));
+    if (err != hipSuccess) return fail_hip("decode attention launch", err);
+    return SENTINEL_HIP_OK;
+}
+
+extern "C" int sentinel_hip_decode_attention_static(const float* query, const float* key_cache, const float* value_cache,
+                                                    float* out, int q_heads, int kv_heads, int head_dim, int cache_stride,
+                                                    int length, float scale, int window_size, int global_token_count,
+                                                    void* stream_ptr) {
+    const char* op = "sentinel_hip_decode_attention_static";
+    const int rc = check_decode(op, query, key_cache, value_cache, out, q_heads, kv_heads, head_dim, cache_stride, length, scale,
+                                global_token_count);
+    if (rc != SENTINEL_HIP_OK) return rc;
+    const size_t need = sentinel_hip_decode_workspace_bytes(q_heads, head_dim, length);
+    if (need > kDecodeStaticScratchBytes)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT,
+                    "%s needs %zu bytes of scratch, the built-in area holds %zu: use sentinel_hip_decode_attention with a "
+                    "workspace of your own",
+                    op, need, (size_t)kDecodeStaticScratchBytes);
+    if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
+    float* scratch = nullptr;  // this device's copy of the array: an address from the runtime, never the array's name
+    hipError_t err = decode_static_scratch_address(&scratch);
+    if (err != hipSuccess) return fail_hip("decode attention scratch lookup", err);
+    // nothing in the area has to start at zero: decode_partial writes every record that decode_merge reads
+    err = launch_decode_attention(query, key_cache, value_cache, out, q_heads, kv_heads, head_dim, cache_stride, length, scale,
+                                  window_size, global_token_count, scratch, static_cast<hipStream_t>(stream_ptr));
     if (err != hipSuccess) return fail_hip("decode attention launch", err);
     return SENTINEL_HIP_OK;
 }

@@ -14,8 +14,36 @@
 #include "flash_common.h"
 
 #include <algorithm>
+#include <mutex>
 
 namespace sentinel_hip {
+
+// Scratch of the entry point that allocates nothing (sentinel_hip_decode_attention_static): the partial
+// (max, sum, acc[d]) records of decode_partial_kernel, in device memory that exists from the moment the code object is
+// loaded.  Every device the library runs on holds its own copy of the array, at its own address, until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress: kernels get the address it returns.
+static __device__ __align__(256) float decode_static_scratch[kDecodeStaticScratchBytes / sizeof(float)];
+
+hipError_t decode_static_scratch_address(float** address) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mutex;
+    static float* per_device[kMaxDevices] = {};
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return err;
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!per_device[device]) {  // first call on this device, with it current: ask the runtime where its copy lives
+        void* found = nullptr;
+        err = hipGetSymbolAddress(&found, HIP_SYMBOL(decode_static_scratch));
+        if (err != hipSuccess) return err;
+        if (!found) return hipErrorInvalidSymbol;
+        per_device[device] = static_cast<float*>(found);
+    }
+    *address = per_device[device];
+    return hipSuccess;
+}
+
 namespace {
 
 constexpr int kDecodeThreads = 256;

@@ -84,6 +84,10 @@ size_t decode_workspace_bytes(int q_heads, int head_dim, int length);
 hipError_t launch_decode_attention(const float* query, const float* key_cache, const float* value_cache, float* out,
                                    int q_heads, int kv_heads, int head_dim, int stride, int length, float scale,
                                    int window, int global_tokens, float* workspace, hipStream_t stream);
+// size of the file-scope device array behind the allocation-free decode entry point, and its address on the current
+// device (looked up once per device)
+constexpr size_t kDecodeStaticScratchBytes = 4u << 20;
+hipError_t decode_static_scratch_address(float** address);
 // in-place rotation of fp32 column-layout rows (tensor already advanced to the first column)
 hipError_t launch_rope_rotate_f32(float* tensor, int heads, int head_dim, int stride_columns, int columns,
                                   int position_offset, int segment_length, const float* cos, const float* sin, bool inverse,

@@ -65,6 +65,8 @@ def load_library():
     lib.sentinel_hip_decode_workspace_bytes.restype = sz
     lib.sentinel_hip_decode_attention.argtypes = [vp] * 4 + [i] * 5 + [f, i, i, vp, sz, vp]
     lib.sentinel_hip_decode_attention.restype = i
+    lib.sentinel_hip_decode_attention_static.argtypes = [vp] * 4 + [i] * 5 + [f, i, i, vp]
+    lib.sentinel_hip_decode_attention_static.restype = i
     lib.sentinel_hip_flash_workspace_bytes.argtypes = [i] * 9
     lib.sentinel_hip_flash_workspace_bytes.restype = sz
     lib.sentinel_hip_flash_max_head_dim.restype = i
