@@ -34,9 +34,34 @@ CONFIGS = {
 SEEDS = {"c1": 1, "c2": 2, "c3": 3, "c4": 4, "c5": 5, "nstar": 6}
 # algorithmic matrix products per kernel (units of B*H*T^2*d FLOPs, causal-halved)
 KERNEL_UNITS = {"fwd_mfma": 2.0, "dkdv_mfma": 4.0, "dq_mfma": 1.0, "fwd_f32": 2.0, "dkdv_f32": 4.0, "dq_f32": 1.0}
-# HBM bytes per launch at the target shape, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-# profiles/nstar_b4_h32_t4096_d128_bf16_counters.txt (scaled by a plain copy kernel of known size: x2.0 / x1.0)
-MEASURED_TRAFFIC_BYTES = {("nstar", "fwd_mfma"): 6.20e8, ("nstar", "dkdv_mfma"): 8.36e8, ("nstar", "dq_mfma"): 9.66e8}
+# kernel names as timed by the library -> the kernel functions they stand for in the profiler's tables
+PROFILED_KERNELS = {"fwd_mfma": ("fwd_mfma_kernel", "fwd_pingpong_kernel"), "dkdv_mfma": ("dkdv_split_kernel", "dkdv_mfma_kernel"),
+                    "dq_mfma": ("dq_mfma_kernel", "dq_pingpong_kernel")}
+COUNTER_SUMMARIES = {"nstar": "nstar_b4_h32_t4096_d128_bf16_counters.txt"}
+
+
+def measured_traffic_bytes(config, kernel):
+    """HBM bytes per launch of `kernel` as measured with rocprofv3 (FETCH_SIZE and WRITE_SIZE runs, scaled by a plain
+    copy kernel of known size): the total_MiB column of the committed counter summary of this workload, or None."""
+    name = COUNTER_SUMMARIES.get(config)
+    if name is None or kernel not in PROFILED_KERNELS:
+        return None
+    try:
+        lines = open(os.path.join(ROOT, "profiles", name)).read().splitlines()
+    except OSError:
+        return None
+    column = None
+    for line in lines:
+        fields = line.split()
+        if "total_MiB" in fields and "FETCH_SIZE" in fields:
+            column = len(fields) - fields.index("total_MiB")  # counted from the right: kernel names hold spaces
+            continue
+        if column is not None and line.startswith(PROFILED_KERNELS[kernel]):
+            try:
+                return float(fields[-column]) * 2 ** 20
+            except (ValueError, IndexError):
+                return None
+    return None
 
 
 def make_inputs(torch, name):
@@ -173,7 +198,7 @@ def cpu_baseline(name, heads_sample):
     }
 
 
-def columns_path(torch, name, steps, rope):
+def columns_path(torch, name, steps, separate):
     """The same step through Sentinel's own tensor layout (fp32 [(head*d + dim), B*T]) with 16-bit arithmetic:
     what the drop-in costs on top of the kernels (layout / type conversion passes, optionally with the rotary
     embedding fused into them instead of four separate elementwise passes)."""
@@ -199,14 +224,18 @@ def columns_path(torch, name, steps, rope):
 
     def step(mode):
         kw = dict(kv_head_count=hkv, compute=dtype, workspace=state["ws"])
-        if mode == "fused":
+        fkw, bkw = {}, {}
+        if mode in ("fused", "fused_kept"):
             kw["rope"] = (cos, sin)
+        if mode in ("plain_kept", "fused_kept"):  # the forward leaves its 16-bit operands in the workspace for the backward
+            fkw, bkw = {"keep_for_backward": True}, {"reuse_forward_workspace": True}
         if mode == "separate":  # the reference's sequence: rotate Q, K in place, attend, rotate dQ, dK back
             HipOps.rotary_rotate_in_place(q, hq, d, d // 2, cos, sin, 0, t)
             HipOps.rotary_rotate_in_place(k, hkv, d, d // 2, cos, sin, 0, t)
-        state["out"], state["lse"] = HipFlashAttention.forward_multi_head(q, k, v, state["out"], state["lse"], *args, **kw)
+        state["out"], state["lse"] = HipFlashAttention.forward_multi_head(q, k, v, state["out"], state["lse"], *args, **kw,
+                                                                          **fkw)
         state["dq"], state["dk"], state["dv"], state["delta"] = HipFlashAttention.backward_multi_head(
-            q, k, v, state["out"], state["lse"], g, state["dq"], state["dk"], state["dv"], state["delta"], *args, **kw)
+            q, k, v, state["out"], state["lse"], g, state["dq"], state["dk"], state["dv"], state["delta"], *args, **kw, **bkw)
         if mode == "separate":
             HipOps.rotary_rotate_inverse_in_place(state["dq"], hq, d, d // 2, cos, sin, 0, t)
             HipOps.rotary_rotate_inverse_in_place(state["dk"], hkv, d, d // 2, cos, sin, 0, t)
@@ -214,7 +243,7 @@ def columns_path(torch, name, steps, rope):
             HipOps.rotary_rotate_inverse_in_place(k, hkv, d, d // 2, cos, sin, 0, t)
 
     report = {}
-    modes = ("plain", "fused", "separate") if rope else ("plain",)
+    modes = ("plain", "plain_kept", "fused", "fused_kept") + (("separate",) if separate else ())
     for mode in modes:
         for _ in range(2):
             step(mode)
@@ -227,7 +256,7 @@ def columns_path(torch, name, steps, rope):
     sentinel_amd.set_kernel_timing(True)
     sentinel_amd.collect_kernel_timings()
     for _ in range(steps):
-        step("fused" if rope else "plain")
+        step("fused_kept")
     times = sentinel_amd.collect_kernel_timings()
     sentinel_amd.set_kernel_timing(False)
     report["kernels_ms"] = {kname: tot / max(n, 1) for kname, (tot, n) in times.items()}
@@ -239,8 +268,13 @@ def columns_path(torch, name, steps, rope):
             # launches mix Q-sized and K/V-sized tensors: count the bytes of all of them
             q_like = 3 + 1  # q, out, d_out in; dq out (+ q in, out out in the forward)
             report[kname + "_avg_ms"] = tot / max(n, 1)
-    report["note"] = ("separate = rotate Q, K in place + plain step + rotate dQ, dK back (+ restoring Q, K: 4 extra passes "
-                      "that a real caller does not need); fused = rotation inside the conversion passes")
+    flops = 7.0 * float(b) * hq * t * t * d
+    for mode in modes:
+        report[mode + "_tflops"] = flops / (report[mode + "_ms_per_step"] * 1e-3) / 1e12
+    report["note"] = ("fp32 [(head*d + dim), B*T] tensors, 16-bit arithmetic; plain = unrotated call; fused = rotary embedding "
+                      "inside the conversion passes; *_kept = the forward call leaves its 16-bit operands in the workspace "
+                      "and the backward call converts d_out only (kernels_ms is this mode); separate = rotate Q, K in place "
+                      "+ plain step + rotate dQ, dK back (+ restoring Q, K: 4 extra passes that a real caller does not need)")
     report["elements_per_q_tensor"] = elems
     return report
 
@@ -357,9 +391,11 @@ def main():
     ap.add_argument("--config", default="nstar", choices=sorted(CONFIGS))
     ap.add_argument("--cpu-heads", type=int, default=8, help="(batch, head) pairs in the CPU baseline sample; 0 = skip")
     ap.add_argument("--no-configs", action="store_true", help="skip the brief timing of the other configurations")
-    ap.add_argument("--columns-path", action="store_true",
-                    help="also time the step through Sentinel's fp32 column layout (conversion passes, fused rotary "
-                         "embedding) and report it under \"columns_path\"")
+    ap.add_argument("--no-columns-path", action="store_true",
+                    help="skip timing the step through Sentinel's fp32 column layout (conversion passes, fused rotary "
+                         "embedding), reported under \"columns_path\"")
+    ap.add_argument("--columns-separate-rope", action="store_true",
+                    help="columns_path also times the reference's sequence of separate in-place rotary passes")
     ap.add_argument("--sparse-path", action="store_true",
                     help="also time the step under sliding-window + global-token masks and report it under \"sparse_path\"")
     ap.add_argument("--decode-path", action="store_true",
@@ -412,7 +448,7 @@ def main():
     dominant = max(counted, key=counted.get)
     achieved = KERNEL_UNITS[dominant] * w.unit_flops / (counted[dominant] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dominant)),
+                "frac": achieved / peak, "traffic": measured_traffic_bytes(args.config, dominant),
                 "kernel_ms": counted[dominant],
                 "algorithmic_flops_per_launch": KERNEL_UNITS[dominant] * w.unit_flops}
 
@@ -462,10 +498,10 @@ def main():
             torch.cuda.empty_cache()
         line["configs"] = others
 
-    if args.columns_path:
+    if not args.no_columns_path and w.dtype != "fp32":
         del w
         torch.cuda.empty_cache()
-        line["columns_path"] = columns_path(torch, args.config, max(args.steps // 5, 3), rope=True)
+        line["columns_path"] = columns_path(torch, args.config, max(args.steps // 5, 3), separate=args.columns_separate_rope)
 
     if args.sparse_path:
         line["sparse_path"] = sparse_path(torch, args.config, max(args.steps // 2, 5))

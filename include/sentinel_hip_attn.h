@@ -71,6 +71,21 @@ enum {
 enum { SENTINEL_HIP_LAYOUT_COLUMNS = 0, SENTINEL_HIP_LAYOUT_BHTD = 1 };
 
 /*
+ * Workspace flags, OR-ed into the `layout` argument. They matter where a workspace is used at all (COLUMNS layout with
+ * MFMA arithmetic) and are ignored elsewhere. The CUDA layer keeps flashLogSumExp from its forward call for its
+ * backward call (CudaCausalSelfAttention.cu:237-249, :421-438); a caller that keeps the workspace the same way saves
+ * the backward four of its conversion passes:
+ *  SENTINEL_HIP_WORKSPACE_KEEP   forward: `workspace` is sized for the BACKWARD call
+ *        (sentinel_hip_flash_workspace_bytes(..., backward = 1)) and the 16-bit copies of q, k, v (rotated, if the call
+ *        rotates) and out are left in it where the backward call looks for them.
+ *  SENTINEL_HIP_WORKSPACE_REUSE  backward: `workspace` is the one a KEEP forward call with the same tensors, geometry,
+ *        mask and rotation filled, untouched since: q, k, v and out are not read or converted again, only d_out is
+ *        (the q / k / v / out pointers are still validated but not dereferenced). Passing a workspace that was not
+ *        filled that way gives wrong gradients: nothing can check it.
+ */
+enum { SENTINEL_HIP_WORKSPACE_KEEP = 0x100, SENTINEL_HIP_WORKSPACE_REUSE = 0x200 };
+
+/*
  * Scratch the caller must provide for a configuration (bytes; 0 when none is needed). Only the
  * COLUMNS layout with MFMA arithmetic needs any (type-converted [B,H,T,d] copies of the operands).
  * `backward` != 0 sizes it for sentinel_hip_flash_bwd, else for sentinel_hip_flash_fwd.

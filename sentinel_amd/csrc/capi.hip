@@ -39,6 +39,8 @@ struct Resolved {
     long long stride;  // column layout only
     int column_start;
     bool adapter;  // column layout fp32 tensors converted to [B,H,T,d] 16-bit for the MFMA kernels
+    bool keep;     // forward: lay the converted operands out where the backward expects them (SENTINEL_HIP_WORKSPACE_KEEP)
+    bool reuse;    // backward: q, k, v, out of the workspace are the forward's (SENTINEL_HIP_WORKSPACE_REUSE)
 };
 
 // Geometry checks shared by both entry points. `op` names the operation in messages.
@@ -47,6 +49,8 @@ int resolve(const char* op, int io_dtype, int compute_dtype, int layout, int q_h
     if (io_dtype < SENTINEL_HIP_F32 || io_dtype > SENTINEL_HIP_F16) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s unknown io dtype %d", op, io_dtype);
     if (compute_dtype < SENTINEL_HIP_COMPUTE_AUTO || compute_dtype > SENTINEL_HIP_COMPUTE_F16)
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s unknown compute dtype %d", op, compute_dtype);
+    const int workspace_flags = layout & (SENTINEL_HIP_WORKSPACE_KEEP | SENTINEL_HIP_WORKSPACE_REUSE);
+    layout &= ~(SENTINEL_HIP_WORKSPACE_KEEP | SENTINEL_HIP_WORKSPACE_REUSE);
     if (layout != SENTINEL_HIP_LAYOUT_COLUMNS && layout != SENTINEL_HIP_LAYOUT_BHTD)
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s unknown layout %d", op, layout);
     if (q_heads <= 0 || head_dim <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s invalid head geometry", op);
@@ -110,6 +114,9 @@ int resolve(const char* op, int io_dtype, int compute_dtype, int layout, int q_h
     r->stride = stride_columns;
     r->column_start = column_start;
     r->adapter = adapter;
+    // without a conversion pass there is nothing to keep: the flags are then accepted and mean nothing
+    r->keep = adapter && (workspace_flags & SENTINEL_HIP_WORKSPACE_KEEP);
+    r->reuse = adapter && (workspace_flags & SENTINEL_HIP_WORKSPACE_REUSE);
     return SENTINEL_HIP_OK;
 }
 
@@ -282,14 +289,15 @@ int flash_fwd(const char* op, const void* q, const void* k, const void* v, void*
     }
 
     // column-layout fp32 tensors: convert operands, run the MFMA kernel, convert the result back
-    const size_t need = workspace_need(r, false);
+    // SENTINEL_HIP_WORKSPACE_KEEP: the workspace is the backward's, and q, out, k, v go where the backward looks for them
+    const size_t need = workspace_need(r, r.keep);
     if (!workspace || workspace_bytes < need || misaligned(workspace))
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s needs %zu bytes of 16-byte aligned workspace", op, need);
     char* ws = static_cast<char*>(workspace);
     void* q16 = ws;
     void* o16 = ws + q_bytes16(g);
-    void* k16 = ws + 2 * q_bytes16(g);
-    void* v16 = ws + 2 * q_bytes16(g) + kv_bytes16(g);
+    void* k16 = ws + (r.keep ? 4 : 2) * q_bytes16(g);
+    void* v16 = static_cast<char*>(k16) + kv_bytes16(g);
     const long long off = r.column_start;
     const int stride = static_cast<int>(r.stride);
     const RopeTables none = {nullptr, nullptr, 0};
@@ -369,19 +377,24 @@ int flash_bwd(const char* op, const void* q, const void* k, const void* v, const
     const int stride = static_cast<int>(r.stride);
     const int T = g.seq_len;
     const RopeTables none = {nullptr, nullptr, 0};
-    hipError_t err = launch_columns_to_bhtd(type, static_cast<const float*>(q) + off, q16, g.q_heads, g.head_dim, stride, T,
-                                            g.packs, rope, stream);
-    if (err == hipSuccess)
-        err = launch_columns_to_bhtd(type, static_cast<const float*>(out) + off, o16, g.q_heads, g.head_dim, stride, T,
-                                     g.packs, none, stream);
+    // SENTINEL_HIP_WORKSPACE_REUSE: q16, o16, k16, v16 are still the ones the forward call left there (rotated Q, K and
+    // the 16-bit O the kernel itself wrote, which is the O that D = rowsum(dO o O) should be formed from anyway)
+    hipError_t err = hipSuccess;
+    if (!r.reuse) {
+        err = launch_columns_to_bhtd(type, static_cast<const float*>(q) + off, q16, g.q_heads, g.head_dim, stride, T, g.packs,
+                                     rope, stream);
+        if (err == hipSuccess)
+            err = launch_columns_to_bhtd(type, static_cast<const float*>(out) + off, o16, g.q_heads, g.head_dim, stride, T,
+                                         g.packs, none, stream);
+        if (err == hipSuccess)
+            err = launch_columns_to_bhtd(type, static_cast<const float*>(k) + off, k16, g.kv_heads, g.head_dim, stride, T,
+                                         g.packs, rope, stream);
+        if (err == hipSuccess)
+            err = launch_columns_to_bhtd(type, static_cast<const float*>(v) + off, v16, g.kv_heads, g.head_dim, stride, T,
+                                         g.packs, none, stream);
+    }
     if (err == hipSuccess)
         err = launch_columns_to_bhtd(type, static_cast<const float*>(d_out) + off, g16, g.q_heads, g.head_dim, stride, T,
-                                     g.packs, none, stream);
-    if (err == hipSuccess)
-        err = launch_columns_to_bhtd(type, static_cast<const float*>(k) + off, k16, g.kv_heads, g.head_dim, stride, T,
-                                     g.packs, rope, stream);
-    if (err == hipSuccess)
-        err = launch_columns_to_bhtd(type, static_cast<const float*>(v) + off, v16, g.kv_heads, g.head_dim, stride, T,
                                      g.packs, none, stream);
     if (err == hipSuccess)
         err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream);

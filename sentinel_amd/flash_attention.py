@@ -25,6 +25,7 @@ OK, INVALID_ARGUMENT, UNSUPPORTED, RUNTIME = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
 COMPUTE_AUTO = -1
 LAYOUT_COLUMNS, LAYOUT_BHTD = 0, 1
+WORKSPACE_KEEP, WORKSPACE_REUSE = 0x100, 0x200  # OR-ed into the layout argument
 
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 _COMPUTE_CODE = {None: COMPUTE_AUTO, "auto": COMPUTE_AUTO, "fp32": F32, "bf16": BF16, "fp16": F16,
@@ -218,8 +219,13 @@ class HipFlashAttention:
     @staticmethod
     def forward_multi_head(query, key, value, out, log_sum_exp, head_count, head_dimension, scale, causal=True,
                            column_start=0, column_count=0, pack_count=1, *, kv_head_count=None, compute=None,
-                           workspace=None, stream=None, rope=None, window_size=0, global_token_count=0):
+                           workspace=None, stream=None, rope=None, window_size=0, global_token_count=0,
+                           keep_for_backward=False):
         """CudaFlashAttention::forwardMultiHead. Returns (out, log_sum_exp) (re-allocated if their shape was wrong).
+
+        keep_for_backward (16-bit arithmetic only): `workspace` must be a tensor sized for the backward call; the
+        converted operands stay in it, and backward_multi_head(..., workspace=the same tensor,
+        reuse_forward_workspace=True) converts d_out only (as the CUDA layer keeps flashLogSumExp between the calls).
 
         window_size / global_token_count: the attention layer's sparse mask (CausalSelfAttention::allowsKey), which
         the CUDA layer can only run on its dense path.
@@ -235,9 +241,12 @@ class HipFlashAttention:
         comp = _COMPUTE_CODE[compute]
         seq = column_count if column_count > 0 else cols - column_start
         ws, ws_bytes, ws_own = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1),
-                                          max(pack_count, 1), False, query.device, workspace)
+                                          max(pack_count, 1), bool(keep_for_backward), query.device, workspace)
+        if keep_for_backward and ws_own is not None:
+            raise ValueError("HipFlashAttention::forwardMultiHead keep_for_backward needs a caller-owned workspace of "
+                             f"at least {ws_bytes} bytes")
         _on_stream(stream, ws_own)
-        tail = (F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start, column_count,
+        tail = (F32, comp, LAYOUT_COLUMNS | (WORKSPACE_KEEP if keep_for_backward else 0), head_count, kv_heads, head_dimension, cols, column_start, column_count,
                 pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes, _stream_handle(stream))
         if window_size > 0 or global_token_count != 0:
             cos, sin, offset = _rope_args(rope, head_dimension) if rope is not None else (None, None, 0)
@@ -262,8 +271,12 @@ class HipFlashAttention:
     def backward_multi_head(query, key, value, out, log_sum_exp, out_gradient, query_gradient, key_gradient,
                             value_gradient, delta_workspace, head_count, head_dimension, scale, causal=True,
                             column_start=0, column_count=0, pack_count=1, *, kv_head_count=None, compute=None,
-                            workspace=None, stream=None, rope=None, window_size=0, global_token_count=0):
+                            workspace=None, stream=None, rope=None, window_size=0, global_token_count=0,
+                            reuse_forward_workspace=False):
         """CudaFlashAttention::backwardMultiHead. Returns (dQ, dK, dV, delta).
+
+        reuse_forward_workspace: `workspace` is the tensor a forward_multi_head(..., keep_for_backward=True) call with
+        the same tensors and arguments filled; query / key / value / out are then not converted again.
 
         rope as in forward_multi_head: query / key unrotated, dQ / dK come back rotated back
         (rotaryRotateInverseInPlace of CudaCausalSelfAttention.cu:508-509 fused into this call)."""
@@ -288,10 +301,13 @@ class HipFlashAttention:
         comp = _COMPUTE_CODE[compute]
         ws, ws_bytes, ws_own = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, max(seq, 1),
                                           packs, True, query.device, workspace)
+        if reuse_forward_workspace and ws_own is not None:
+            raise ValueError("HipFlashAttention::backwardMultiHead reuse_forward_workspace needs the forward call's workspace")
         _on_stream(stream, ws_own)
         head = (_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp), _ptr(out_gradient), _ptr(query_gradient),
                 _ptr(key_gradient), _ptr(value_gradient), _ptr(delta_workspace))
-        tail = (F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension, cols, column_start, column_count,
+        tail = (F32, comp, LAYOUT_COLUMNS | (WORKSPACE_REUSE if reuse_forward_workspace else 0), head_count, kv_heads,
+                head_dimension, cols, column_start, column_count,
                 pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes, _stream_handle(stream))
         if window_size > 0 or global_token_count != 0:
             cos, sin, offset = _rope_args(rope, head_dimension) if rope is not None else (None, None, 0)

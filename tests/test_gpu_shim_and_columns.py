@@ -73,3 +73,43 @@ def test_unsupported_head_dim_is_reported_not_faked():
     # the exact fp32 kernels take any head_dim <= 128
     out, lse = HipFlashAttention.forward_multi_head(q + 0.01, q, q, None, None, 4, 48, 0.1)
     assert torch.isfinite(out).all()
+
+
+@pytest.mark.parametrize("variant", ["plain", "rope", "sparse_rope"])
+def test_backward_reuses_the_forward_workspace(variant):
+    """SENTINEL_HIP_WORKSPACE_KEEP / _REUSE: the forward call leaves its 16-bit operands in the caller's workspace and
+    the backward call converts d_out only.  Same kernels on the same 16-bit operands: gradients identical to the plain
+    pair of calls, bit for bit, even when the fp32 q / k / v / out handed to the backward call are garbage."""
+    import oracle_lib
+    import sentinel_amd
+    from sentinel_amd import HipFlashAttention
+    hq, hkv, d, t, packs, col0, pad = 8, 2, 128, 200, 2, 4, 4
+    print(f"case workspace reuse {variant}", flush=True)
+    q, k, v, g = gpu_util.make_inputs(hq, hkv, d, t, packs, seed=77, dtype="bf16", col0=col0, pad=pad)
+    qd, kd, vd, gd = (torch.from_numpy(x).cuda() for x in (q, k, v, g))
+    scale = 1.0 / np.sqrt(np.float32(d))
+    args = (hq, d, scale, True, col0, t, packs)
+    kw = dict(kv_head_count=hkv, compute="bf16")
+    if "rope" in variant:
+        cos, sin = oracle_lib.rope_tables(d, t)
+        kw["rope"] = (torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda())
+    if "sparse" in variant:
+        kw.update(window_size=60, global_token_count=3)
+    out0, lse0 = HipFlashAttention.forward_multi_head(qd, kd, vd, None, None, *args, **kw)
+    dq0, dk0, dv0, _ = HipFlashAttention.backward_multi_head(qd, kd, vd, out0, lse0, gd, None, None, None, None, *args, **kw)
+
+    lib = sentinel_amd.load_library()
+    need = lib.sentinel_hip_flash_workspace_bytes(0, 1, 0, hq, hkv, d, t, packs, 1)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    out1, lse1 = HipFlashAttention.forward_multi_head(qd, kd, vd, None, None, *args, workspace=ws, keep_for_backward=True, **kw)
+    junk_q, junk_k, junk_v, junk_o = (torch.full_like(x, float("nan")) for x in (qd, kd, vd, out1))
+    dq1, dk1, dv1, _ = HipFlashAttention.backward_multi_head(junk_q, junk_k, junk_v, junk_o, lse1, gd, None, None, None, None,
+                                                             *args, workspace=ws, reuse_forward_workspace=True, **kw)
+    torch.cuda.synchronize()
+    inside = torch.zeros(qd.shape[1], dtype=torch.bool, device="cuda")
+    inside[col0:col0 + packs * t] = True
+    for name, a, b in (("out", out0, out1), ("lse", lse0, lse1), ("dq", dq0, dq1), ("dk", dk0, dk1), ("dv", dv0, dv1)):
+        assert torch.equal(a[:, inside], b[:, inside]), f"{name} differs with the kept workspace"
+    # a workspace that is too small for the backward is refused, not silently replaced
+    with pytest.raises(ValueError, match="keep_for_backward needs"):
+        HipFlashAttention.forward_multi_head(qd, kd, vd, None, None, *args, workspace=ws[:need // 2], keep_for_backward=True, **kw)
