@@ -18,8 +18,16 @@
 // in place of attendCachedQuery's per-head copies and GEMMs (:318-341).
 // Layers with a sliding window / global tokens (windowSize, globalTokenCount) run on the same kernels with the
 // sparse mask (sentinel_hip_flash_fwd_sparse / _bwd_sparse), where the CUDA class falls back to its dense path.
-// Not built: that dense materialising fallback itself (preferFlashAttention = false throws std::runtime_error
-// instead of running something else).
+// With preferFlashAttention = false the layer takes the dense materialising path (Cuda/CudaCausalSelfAttention.cu:255-314
+// forward, :445-505 backward): keys x queries scores per (head, pack), probabilities cached for the backward. The CUDA
+// class walks the heads one at a time (three head copies, GEMM, scale, mask, softmax, copy, GEMM, head write-back per
+// head); here the head blocks of the [(head*d + dim), column] matrices are addressed in place by strided-batched
+// GEMMs over all K/V heads at once and one fused scale + mask + softmax launch covers every head and pack.
+// Multi-head layers (kvHeadCount == headCount) keep the three projection weights stacked in qkvWeight
+// (usesFusedQkv, :19-21, :190-201): one projection GEMM forward, one weight-gradient and one input-gradient GEMM
+// backward. queryWeight / keyWeight / valueWeight, query / key / value and the three gradients are row-block views of
+// the stacked matrices, so the CUDA class's device-to-device split copies and its syncFusedQkvWeight re-stacking after
+// an optimizer step have nothing left to do.
 // Link against libsentinel_hip_attn.so, rocBLAS and the HIP runtime.
 #ifndef SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
 #define SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
@@ -61,6 +69,28 @@ public:
             static_cast<rocblas_int>(b.cols), a.buffer.deviceData, static_cast<rocblas_int>(a.cols), &beta,
             c.buffer.deviceData, static_cast<rocblas_int>(n));
         if (st != rocblas_status_success) throw std::runtime_error("HipGemm rocblas_sgemm failed");
+    }
+
+    /// `batch` products C_i = op(A_i) op(B_i) (+ C_i) on row-major fp32 blocks addressed in place: block i of X starts
+    /// at x + i * strideX and its rows are ldX floats apart. op(A) is m x k, op(B) is k x n. Head blocks of the
+    /// [(head*d + dim), column] activations are such blocks (stride = d * columns, ld = columns), which is what lets
+    /// the dense attention path run without CudaOps::extractHeadInto / writeHead copies.
+    static void multiplyBatched(const float* a, size_t lda, long long strideA, bool transposeA, const float* b, size_t ldb,
+                                long long strideB, bool transposeB, float* c, size_t ldc, long long strideC, size_t m, size_t n,
+                                size_t k, int batch, bool accumulate = false) {
+        if (!a || !b || !c || m == 0 || n == 0 || k == 0 || batch <= 0)
+            throw std::invalid_argument("HipGemm::multiplyBatched empty operand");
+        const float alpha = 1.0f;
+        const float beta = accumulate ? 1.0f : 0.0f;
+        rocblas_handle h = handle();
+        if (rocblas_set_stream(h, HipFlashAttention::activeStream()) != rocblas_status_success)
+            throw std::runtime_error("HipGemm rocblas_set_stream failed");
+        const rocblas_status st = rocblas_sgemm_strided_batched(
+            h, transposeB ? rocblas_operation_transpose : rocblas_operation_none,
+            transposeA ? rocblas_operation_transpose : rocblas_operation_none, static_cast<rocblas_int>(n),
+            static_cast<rocblas_int>(m), static_cast<rocblas_int>(k), &alpha, b, static_cast<rocblas_int>(ldb), strideB, a,
+            static_cast<rocblas_int>(lda), strideA, &beta, c, static_cast<rocblas_int>(ldc), strideC, batch);
+        if (st != rocblas_status_success) throw std::runtime_error("HipGemm rocblas_sgemm_strided_batched failed");
     }
 
 private:
@@ -144,6 +174,9 @@ private:
 class HipCausalSelfAttention {
 public:
     HipMatrix queryWeight, keyWeight, valueWeight, outputWeight;
+    /// stacked [query; key; value] weights, projections and gradients of a multi-head layer (usesFusedQkv); the split
+    /// matrices above and below are then views of their row blocks
+    HipMatrix qkvWeight, qkvProjected, qkvGradient, qkvWeightGradient;
     HipMatrix cosTable, sinTable;
     int headCount = 0;
     int kvHeadCount = 0;
@@ -160,6 +193,11 @@ public:
     HipMatrix query, key, value, attended, output;
     HipMatrix inputCache, attendedGradient, queryGradient, keyGradient, valueGradient;
     HipMatrix flashLogSumExp, flashDelta;
+    /// dense path: probabilities of every (head, pack), row (head * packs + pack) holds one keys x queries matrix; kept
+    /// for the backward like the CUDA class's cachedHeadProbabilities
+    HipMatrix probabilities;
+    /// dense path backward: probability / score gradients of the heads one batched product covers
+    HipMatrix scoreGradient;
     HipDeviceBuffer decodeWorkspace;
 
     /// upload weights and build the RoPE tables the way RotaryEmbedding does (Layers/RotaryEmbedding.cpp:8-29)
@@ -179,6 +217,21 @@ public:
         globalTokenCount = host.globalTokenCount;
         const size_t e = static_cast<size_t>(host.embeddingDim);
         const size_t qRows = static_cast<size_t>(headCount) * headDimension, kvRows = static_cast<size_t>(kv) * headDimension;
+        if (host.queryWeight.size() != qRows * e || host.keyWeight.size() != kvRows * e || host.valueWeight.size() != kvRows * e)
+            throw std::invalid_argument(std::string(op) + " key/value rows mismatch kvHeadCount");
+        // views of a previous configuration's stacked matrices must not outlive them
+        HipMatrix* mayBeViews[] = {&queryWeight, &keyWeight, &valueWeight, &query, &key, &value, &queryGradient, &keyGradient,
+                                   &valueGradient};
+        for (HipMatrix* m : mayBeViews)
+            if (!m->buffer.ownsMemory) *m = HipMatrix();
+        if (usesFusedQkv()) {
+            qkvWeight.ensureSize(3 * qRows, e);
+            queryWeight.viewRows(qkvWeight, 0, qRows);
+            keyWeight.viewRows(qkvWeight, qRows, qRows);
+            valueWeight.viewRows(qkvWeight, 2 * qRows, qRows);
+        } else {
+            qkvWeight = HipMatrix();
+        }
         queryWeight.upload(host.queryWeight, qRows, e);
         keyWeight.upload(host.keyWeight, kvRows, e);
         valueWeight.upload(host.valueWeight, kvRows, e);
@@ -199,6 +252,59 @@ public:
         HipCausalSelfAttention layer;
         layer.uploadFrom(host);
         return layer;
+    }
+
+    /// one stacked projection for multi-head layers (CudaCausalSelfAttention::usesFusedQkv, Cuda/CudaCausalSelfAttention.cu:19-21)
+    bool usesFusedQkv() const { return kvHeadCount > 0 && kvHeadCount == headCount; }
+
+    /// CudaCausalSelfAttention::syncFusedQkvWeight (:155-173) re-stacks the split weights after the optimizer changed
+    /// them. Here the split weights are views of the stacked matrix, so an update of either is an update of both and
+    /// there is nothing to copy; only split weights that were replaced by matrices of their own are stacked again.
+    void syncFusedQkvWeight() {
+        if (!usesFusedQkv()) {
+            qkvWeight = HipMatrix();
+            return;
+        }
+        if (queryWeight.empty() || keyWeight.empty() || valueWeight.empty()) return;
+        if (queryWeight.cols != keyWeight.cols || queryWeight.cols != valueWeight.cols)
+            throw std::invalid_argument("HipCausalSelfAttention::syncFusedQkvWeight embed mismatch");
+        if (queryWeight.rows != keyWeight.rows || queryWeight.rows != valueWeight.rows)
+            throw std::invalid_argument("HipCausalSelfAttention::syncFusedQkvWeight projection rows mismatch");
+        const size_t rows = queryWeight.rows;
+        const bool stacked = !qkvWeight.empty() && qkvWeight.rows == 3 * rows && qkvWeight.cols == queryWeight.cols &&
+                             queryWeight.buffer.deviceData == qkvWeight.buffer.deviceData &&
+                             keyWeight.buffer.deviceData == qkvWeight.buffer.deviceData + rows * qkvWeight.cols &&
+                             valueWeight.buffer.deviceData == qkvWeight.buffer.deviceData + 2 * rows * qkvWeight.cols;
+        if (stacked) return;
+        HipMatrix fresh;
+        fresh.ensureSize(3 * rows, queryWeight.cols);
+        HipMatrix* parts[3] = {&queryWeight, &keyWeight, &valueWeight};
+        for (int i = 0; i < 3; ++i)
+            throwIfHipFailed(hipMemcpyAsync(fresh.buffer.deviceData + i * rows * fresh.cols, parts[i]->buffer.deviceData,
+                                            parts[i]->byteCount(), hipMemcpyDeviceToDevice, HipFlashAttention::activeStream()),
+                             "HipCausalSelfAttention::syncFusedQkvWeight copy");
+        throwIfHipFailed(hipStreamSynchronize(HipFlashAttention::activeStream()), "HipCausalSelfAttention::syncFusedQkvWeight");
+        qkvWeight = std::move(fresh);
+        for (int i = 0; i < 3; ++i) parts[i]->viewRows(qkvWeight, i * rows, rows);
+    }
+
+    /// release dense-only scratch (CudaCausalSelfAttention::releaseDenseAttentionScratch, :59-77)
+    void releaseDenseAttentionScratch() {
+        probabilities = HipMatrix();
+        scoreGradient = HipMatrix();
+    }
+    /// release flash-only scratch (CudaCausalSelfAttention::releaseFlashAttentionScratch, :79-86)
+    void releaseFlashAttentionScratch() {
+        flashLogSumExp = HipMatrix();
+        flashDelta = HipMatrix();
+    }
+    /// free the activations after a forward, weights kept (CudaCausalSelfAttention::releaseActivationScratch, :88-108)
+    void releaseActivationScratch() {
+        releaseFlashAttentionScratch();
+        releaseDenseAttentionScratch();
+        HipMatrix* all[] = {&query, &key, &value, &queryGradient, &keyGradient, &valueGradient, &qkvProjected, &qkvGradient,
+                            &attended, &output, &inputCache, &attendedGradient};
+        for (HipMatrix* m : all) *m = HipMatrix();
     }
 
     /// CudaCausalSelfAttention::canUseFlashAttention (Cuda/CudaCausalSelfAttention.cu:46-57) without the
@@ -224,22 +330,24 @@ public:
         if (segmentLength <= 0) segmentLength = columns;
         if (columns % segmentLength != 0) throw std::invalid_argument(std::string(op) + " columns must be a multiple of segmentLength");
         if (segmentLength > maximumPositionCount) throw std::invalid_argument(std::string(op) + " segmentLength exceeds RoPE table");
-        if (!canUseFlashAttention(segmentLength))
-            throw std::runtime_error(std::string(op) + " needs the dense attention path (flash disabled), which is not built");
         activeSegmentLength = segmentLength;
         activePackCount = columns / segmentLength;
-        usedFlashAttention = true;
+        usedFlashAttention = canUseFlashAttention(segmentLength);
 
         inputCache.ensureSize(input.rows, input.cols);
         throwIfHipFailed(hipMemcpyAsync(inputCache.buffer.deviceData, input.buffer.deviceData, input.byteCount(),
                                         hipMemcpyDeviceToDevice, HipFlashAttention::activeStream()),
                          "HipCausalSelfAttention::forward input copy");
-        HipGemm::multiplyInto(queryWeight, input, query);
-        HipGemm::multiplyInto(keyWeight, input, key);
-        HipGemm::multiplyInto(valueWeight, input, value);
+        project(input);
         const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
         const bool sparse = usesSparseMask(segmentLength);
-        if (fusedRotation()) {
+        if (!usedFlashAttention) {
+            releaseFlashAttentionScratch();
+            HipOps::rotaryRotateInPlace(query, headCount, headDimension, pairCount, cosTable, sinTable, 0, segmentLength);
+            HipOps::rotaryRotateInPlace(key, kvHeadCount, headDimension, pairCount, cosTable, sinTable, 0, segmentLength);
+            attendDense(segmentLength, activePackCount);
+        } else if (fusedRotation()) {
+            releaseDenseAttentionScratch();
             if (sparse)
                 HipFlashAttention::forwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, &cosTable, &sinTable, 0,
                                                           windowSize, globalTokenCount, headCount, headDimension, scale, 0,
@@ -249,6 +357,7 @@ public:
                                                         headCount, headDimension, scale, true, 0, segmentLength,
                                                         activePackCount, kvHeadCount);
         } else {
+            releaseDenseAttentionScratch();
             HipOps::rotaryRotateInPlace(query, headCount, headDimension, pairCount, cosTable, sinTable, 0, segmentLength);
             HipOps::rotaryRotateInPlace(key, kvHeadCount, headDimension, pairCount, cosTable, sinTable, 0, segmentLength);
             if (sparse)
@@ -262,18 +371,39 @@ public:
         HipGemm::multiplyInto(outputWeight, attended, out);
     }
 
-    /// backprop through the layer; weight gradients are overwritten (summed over all columns of the batch)
+    /// backprop through the layer; weight gradients are overwritten (summed over all columns of the batch).
+    /// materializeSplitWeightGrads = false leaves the stacked qkvWeightGradient only (multi-head layers), as in
+    /// CudaCausalSelfAttention::backward (Cuda/CudaCausalSelfAttention.cu:357-365, :519-529).
     void backward(const HipMatrix& outputGradient, HipMatrix& inputGradient, HipMatrix& queryWeightGradient,
-                  HipMatrix& keyWeightGradient, HipMatrix& valueWeightGradient, HipMatrix& outputWeightGradient) {
+                  HipMatrix& keyWeightGradient, HipMatrix& valueWeightGradient, HipMatrix& outputWeightGradient,
+                  bool materializeSplitWeightGrads = true) {
         const char* op = "HipCausalSelfAttention::backward";
-        if (inputCache.empty() || !usedFlashAttention) throw std::logic_error(std::string(op) + " called before forward");
+        if (inputCache.empty()) throw std::logic_error(std::string(op) + " called before forward");
         if (outputGradient.rows != outputWeight.rows || outputGradient.cols != attended.cols)
             throw std::invalid_argument(std::string(op) + " output gradient shape mismatch");
+        if (usedFlashAttention) {
+            if (flashLogSumExp.rows != static_cast<size_t>(headCount) || flashLogSumExp.cols != query.cols)
+                throw std::invalid_argument(std::string(op) + " flash logSumExp shape mismatch");
+        } else if (probabilities.rows != static_cast<size_t>(headCount) * activePackCount) {
+            throw std::invalid_argument(std::string(op) + " head cache size mismatch");
+        }
         HipGemm::multiplyInto(outputGradient, attended, outputWeightGradient, false, true);
         HipGemm::multiplyInto(outputWeight, outputGradient, attendedGradient, true, false);
+        if (usesFusedQkv()) {
+            qkvGradient.ensureSize(3 * query.rows, query.cols);
+            queryGradient.viewRows(qkvGradient, 0, query.rows);
+            keyGradient.viewRows(qkvGradient, query.rows, query.rows);
+            valueGradient.viewRows(qkvGradient, 2 * query.rows, query.rows);
+        }
         const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
         const bool sparse = usesSparseMask(activeSegmentLength);
-        if (fusedRotation()) {
+        if (!usedFlashAttention) {
+            backwardDense(activeSegmentLength, activePackCount);
+            HipOps::rotaryRotateInverseInPlace(queryGradient, headCount, headDimension, pairCount, cosTable, sinTable, 0,
+                                               activeSegmentLength);
+            HipOps::rotaryRotateInverseInPlace(keyGradient, kvHeadCount, headDimension, pairCount, cosTable, sinTable, 0,
+                                               activeSegmentLength);
+        } else if (fusedRotation()) {
             if (sparse)
                 HipFlashAttention::backwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, attendedGradient,
                                                            queryGradient, keyGradient, valueGradient, flashDelta, &cosTable,
@@ -300,12 +430,33 @@ public:
             HipOps::rotaryRotateInverseInPlace(keyGradient, kvHeadCount, headDimension, pairCount, cosTable, sinTable, 0,
                                                activeSegmentLength);
         }
-        HipGemm::multiplyInto(queryGradient, inputCache, queryWeightGradient, false, true);
-        HipGemm::multiplyInto(keyGradient, inputCache, keyWeightGradient, false, true);
-        HipGemm::multiplyInto(valueGradient, inputCache, valueWeightGradient, false, true);
-        HipGemm::multiplyInto(queryWeight, queryGradient, inputGradient, true, false);
-        HipGemm::multiplyInto(keyWeight, keyGradient, inputGradient, true, false, true);
-        HipGemm::multiplyInto(valueWeight, valueGradient, inputGradient, true, false, true);
+        if (usesFusedQkv()) {
+            if (queryGradient.buffer.deviceData != qkvGradient.buffer.deviceData)
+                throw std::logic_error(std::string(op) + " gradient views were replaced");
+            // stacked [dQ; dK; dV]: one weight-gradient product and one input-gradient product (:507-530)
+            HipGemm::multiplyInto(qkvGradient, inputCache, qkvWeightGradient, false, true);
+            if (materializeSplitWeightGrads) {
+                HipMatrix* parts[3] = {&queryWeightGradient, &keyWeightGradient, &valueWeightGradient};
+                for (int i = 0; i < 3; ++i) {
+                    parts[i]->ensureSize(queryWeight.rows, queryWeight.cols);
+                    throwIfHipFailed(hipMemcpyAsync(parts[i]->buffer.deviceData,
+                                                    qkvWeightGradient.buffer.deviceData + i * queryWeight.elementCount(),
+                                                    queryWeight.byteCount(), hipMemcpyDeviceToDevice,
+                                                    HipFlashAttention::activeStream()),
+                                     "HipCausalSelfAttention::backward weight gradient split");
+                }
+            }
+            HipGemm::multiplyInto(qkvWeight, qkvGradient, inputGradient, true, false);
+        } else {
+            if (materializeSplitWeightGrads) {
+                HipGemm::multiplyInto(queryGradient, inputCache, queryWeightGradient, false, true);
+                HipGemm::multiplyInto(keyGradient, inputCache, keyWeightGradient, false, true);
+                HipGemm::multiplyInto(valueGradient, inputCache, valueWeightGradient, false, true);
+            }
+            HipGemm::multiplyInto(queryWeight, queryGradient, inputGradient, true, false);
+            HipGemm::multiplyInto(keyWeight, keyGradient, inputGradient, true, false, true);
+            HipGemm::multiplyInto(valueWeight, valueGradient, inputGradient, true, false, true);
+        }
     }
 
     /// reset cache then run full sequence attention and append rotated KV
@@ -316,13 +467,13 @@ public:
         if (queryWeight.cols != input.rows) throw std::invalid_argument(std::string(op) + " embedding dim mismatch");
         if (static_cast<int>(input.cols) > maximumPositionCount)
             throw std::invalid_argument(std::string(op) + " sequence longer than maximumPositionCount");
-        if (!canUseFlashAttention(static_cast<int>(input.cols)))
-            throw std::runtime_error(std::string(op) + " needs the dense attention path (flash disabled), which is not built");
         cache.ensureCapacity(static_cast<int>(keyWeight.rows), maximumPositionCount);
         projectAndRotate(input, 0);
         cache.append(key, value);
         const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
-        if (usesSparseMask(static_cast<int>(input.cols)))
+        if (!canUseFlashAttention(static_cast<int>(input.cols)))
+            attendDense(static_cast<int>(input.cols), 1);
+        else if (usesSparseMask(static_cast<int>(input.cols)))
             HipFlashAttention::forwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, nullptr, nullptr, 0, windowSize,
                                                       globalTokenCount, headCount, headDimension, scale, 0,
                                                       static_cast<int>(input.cols), 1, kvHeadCount);
@@ -348,14 +499,93 @@ public:
     }
 
 private:
-    // Q, K, V projections of the input columns, Q and K rotated in place for positions offset, offset + 1, ...
-    // (CudaCausalSelfAttention::projectAndRotate, Cuda/CudaCausalSelfAttention.cu:181-208)
+    // Q, K, V projections of the input columns: one stacked product whose row blocks query / key / value then view
+    // (multi-head layers), three products otherwise (CudaCausalSelfAttention::projectAndRotate,
+    // Cuda/CudaCausalSelfAttention.cu:181-208, without its three split copies)
+    void project(const HipMatrix& input) {
+        if (usesFusedQkv()) {
+            syncFusedQkvWeight();
+            HipGemm::multiplyInto(qkvWeight, input, qkvProjected);
+            query.viewRows(qkvProjected, 0, queryWeight.rows);
+            key.viewRows(qkvProjected, queryWeight.rows, queryWeight.rows);
+            value.viewRows(qkvProjected, 2 * queryWeight.rows, queryWeight.rows);
+        } else {
+            HipGemm::multiplyInto(queryWeight, input, query);
+            HipGemm::multiplyInto(keyWeight, input, key);
+            HipGemm::multiplyInto(valueWeight, input, value);
+        }
+    }
+
+    // projections, then Q and K rotated in place for positions offset, offset + 1, ...
     void projectAndRotate(const HipMatrix& input, int positionOffset) {
-        HipGemm::multiplyInto(queryWeight, input, query);
-        HipGemm::multiplyInto(keyWeight, input, key);
-        HipGemm::multiplyInto(valueWeight, input, value);
+        project(input);
         HipOps::rotaryRotateInPlace(query, headCount, headDimension, pairCount, cosTable, sinTable, positionOffset);
         HipOps::rotaryRotateInPlace(key, kvHeadCount, headDimension, pairCount, cosTable, sinTable, positionOffset);
+    }
+
+    // Dense forward (Cuda/CudaCausalSelfAttention.cu:255-314): P = softmax(mask(scale * K^T Q)) per (head, pack), kept in
+    // `probabilities`; attended = V P. Head h of query head group j of K/V head v is h = v * group + j: for a fixed
+    // (pack, j) the blocks of the K/V heads are a constant stride apart in every operand, one batched product each.
+    void attendDense(int segmentLength, int packCount) {
+        const size_t t = static_cast<size_t>(segmentLength), cols = query.cols, d = static_cast<size_t>(headDimension);
+        const size_t tt = t * t;
+        const int group = headCount / kvHeadCount;
+        const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
+        probabilities.ensureSize(static_cast<size_t>(headCount) * packCount, tt);
+        attended.ensureSize(query.rows, cols);
+        float* p = probabilities.buffer.deviceData;
+        const long long kvStride = static_cast<long long>(d * cols), qStride = kvStride * group;
+        const long long pStride = static_cast<long long>(tt) * packCount * group;
+        for (int pack = 0; pack < packCount; ++pack)
+            for (int j = 0; j < group; ++j) {
+                const size_t c0 = static_cast<size_t>(pack) * t;
+                HipGemm::multiplyBatched(key.buffer.deviceData + c0, cols, kvStride, true,
+                                         query.buffer.deviceData + j * d * cols + c0, cols, qStride, false,
+                                         p + (static_cast<size_t>(j) * packCount + pack) * tt, t, pStride, t, t, d, kvHeadCount);
+            }
+        HipOps::maskedSoftmaxInPlace(p, headCount * packCount, static_cast<long long>(tt), segmentLength, segmentLength, scale,
+                                     windowSize, globalTokenCount);
+        for (int pack = 0; pack < packCount; ++pack)
+            for (int j = 0; j < group; ++j) {
+                const size_t c0 = static_cast<size_t>(pack) * t;
+                HipGemm::multiplyBatched(value.buffer.deviceData + c0, cols, kvStride, false,
+                                         p + (static_cast<size_t>(j) * packCount + pack) * tt, t, pStride, false,
+                                         attended.buffer.deviceData + j * d * cols + c0, cols, qStride, d, t, t, kvHeadCount);
+            }
+    }
+
+    // Dense backward (:445-505) from the cached probabilities: per (pack, j) and batched over the K/V heads
+    //   dV += dA P^T,  dP = V^T dA,  dS = scale * P (dP - colsum(dP P)) masked,  dQ = K dS,  dK += Q dS^T
+    // (+= over the query heads j of a K/V head: the first j overwrites, so no zero pass is needed).
+    void backwardDense(int segmentLength, int packCount) {
+        const size_t t = static_cast<size_t>(segmentLength), cols = query.cols, d = static_cast<size_t>(headDimension);
+        const size_t tt = t * t;
+        const int group = headCount / kvHeadCount;
+        const float scale = 1.0f / std::sqrt(static_cast<float>(headDimension));
+        queryGradient.ensureSize(query.rows, cols);
+        keyGradient.ensureSize(key.rows, cols);
+        valueGradient.ensureSize(value.rows, cols);
+        scoreGradient.ensureSize(static_cast<size_t>(kvHeadCount), tt);
+        float* ds = scoreGradient.buffer.deviceData;
+        const long long kvStride = static_cast<long long>(d * cols), qStride = kvStride * group;
+        const long long pStride = static_cast<long long>(tt) * packCount * group, dsStride = static_cast<long long>(tt);
+        for (int pack = 0; pack < packCount; ++pack)
+            for (int j = 0; j < group; ++j) {
+                const size_t c0 = static_cast<size_t>(pack) * t;
+                const float* p = probabilities.buffer.deviceData + (static_cast<size_t>(j) * packCount + pack) * tt;
+                const float* dA = attendedGradient.buffer.deviceData + j * d * cols + c0;
+                const float* q = query.buffer.deviceData + j * d * cols + c0;
+                HipGemm::multiplyBatched(dA, cols, qStride, false, p, t, pStride, true, valueGradient.buffer.deviceData + c0, cols,
+                                         kvStride, d, t, t, kvHeadCount, j > 0);
+                HipGemm::multiplyBatched(value.buffer.deviceData + c0, cols, kvStride, true, dA, cols, qStride, false, ds, t,
+                                         dsStride, t, t, d, kvHeadCount);
+                HipOps::maskedSoftmaxBackwardInPlace(p, pStride, ds, dsStride, kvHeadCount, segmentLength, segmentLength, scale,
+                                                     windowSize, globalTokenCount);
+                HipGemm::multiplyBatched(key.buffer.deviceData + c0, cols, kvStride, false, ds, t, dsStride, false,
+                                         queryGradient.buffer.deviceData + j * d * cols + c0, cols, qStride, d, t, t, kvHeadCount);
+                HipGemm::multiplyBatched(q, cols, qStride, false, ds, t, dsStride, true, keyGradient.buffer.deviceData + c0, cols,
+                                         kvStride, d, t, t, kvHeadCount, j > 0);
+            }
     }
 
     void attendCachedQuery(const HipKvCache& cache, HipMatrix& out) {

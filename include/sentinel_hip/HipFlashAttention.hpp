@@ -26,27 +26,33 @@ inline void throwIfHipFailed(hipError_t status, const char* what) {
     if (status != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(status));
 }
 
-/// reusable device float buffer, grows only when capacity is too small
+/// reusable device float buffer, grows only when capacity is too small; it can also stand for a range of another
+/// buffer's memory (alias), which it then never frees
 class HipDeviceBuffer {
 public:
     float* deviceData = nullptr;
     size_t capacityBytes = 0;
+    bool ownsMemory = true;
 
     HipDeviceBuffer() = default;
     ~HipDeviceBuffer() { this->free(); }
     HipDeviceBuffer(const HipDeviceBuffer&) = delete;
     HipDeviceBuffer& operator=(const HipDeviceBuffer&) = delete;
-    HipDeviceBuffer(HipDeviceBuffer&& other) noexcept : deviceData(other.deviceData), capacityBytes(other.capacityBytes) {
+    HipDeviceBuffer(HipDeviceBuffer&& other) noexcept
+        : deviceData(other.deviceData), capacityBytes(other.capacityBytes), ownsMemory(other.ownsMemory) {
         other.deviceData = nullptr;
         other.capacityBytes = 0;
+        other.ownsMemory = true;
     }
     HipDeviceBuffer& operator=(HipDeviceBuffer&& other) noexcept {
         if (this != &other) {
             this->free();
             deviceData = other.deviceData;
             capacityBytes = other.capacityBytes;
+            ownsMemory = other.ownsMemory;
             other.deviceData = nullptr;
             other.capacityBytes = 0;
+            other.ownsMemory = true;
         }
         return *this;
     }
@@ -56,10 +62,18 @@ public:
         throwIfHipFailed(hipMalloc(reinterpret_cast<void**>(&deviceData), requiredBytes), "HipDeviceBuffer hipMalloc");
         capacityBytes = requiredBytes;
     }
+    /// stand for `bytes` of memory that someone else owns and keeps alive
+    void alias(float* memory, size_t bytes) {
+        this->free();
+        deviceData = memory;
+        capacityBytes = bytes;
+        ownsMemory = false;
+    }
     void free() {
-        if (deviceData) (void)hipFree(deviceData);
+        if (deviceData && ownsMemory) (void)hipFree(deviceData);
         deviceData = nullptr;
         capacityBytes = 0;
+        ownsMemory = true;
     }
 };
 
@@ -94,6 +108,14 @@ public:
         return host;
     }
     void fill(float value) { upload(std::vector<float>(elementCount(), value), rows, cols); }
+    /// become rows [firstRow, firstRow + rowCount) of `whole` without a copy: a block of rows of a row-major matrix is
+    /// itself a row-major matrix. `whole` must outlive the view and keep its size.
+    void viewRows(HipMatrix& whole, size_t firstRow, size_t rowCount) {
+        if (firstRow + rowCount > whole.rows) throw std::invalid_argument("HipMatrix::viewRows outside the matrix");
+        rows = rowCount;
+        cols = whole.cols;
+        buffer.alias(whole.buffer.deviceData + firstRow * whole.cols, byteCount());
+    }
 };
 
 class HipFlashAttention {
@@ -365,7 +387,33 @@ public:
                positionOffset, segmentLength, 1);
     }
 
+    /// CudaOps::scaleInPlace + applySparseAttentionMaskInPlace + softmaxInto (Cuda/CudaOps.hpp:141-147) for `batch`
+    /// keys x queries score matrices, `batchStride` floats apart, in place and in one launch
+    static void maskedSoftmaxInPlace(float* scores, int batch, long long batchStride, int keyCount, int queryCount, float scale,
+                                     int windowSize, int globalTokenCount, int queryPositionStart = 0, int segmentLength = 0) {
+        throwUnlessOk(sentinel_hip_dense_softmax_fwd(scores, batch, batchStride, keyCount, queryCount, queryPositionStart,
+                                                     windowSize, globalTokenCount, segmentLength, scale,
+                                                     HipFlashAttention::activeStream()));
+    }
+    /// CudaOps::softmaxBackwardInto + zeroForbiddenScoreGradientsInPlace + scaleInPlace (Cuda/CudaOps.hpp:150-153): the
+    /// score gradient replaces the probability gradient
+    static void maskedSoftmaxBackwardInPlace(const float* probabilities, long long probabilityBatchStride, float* gradient,
+                                             long long gradientBatchStride, int batch, int keyCount, int queryCount, float scale,
+                                             int windowSize, int globalTokenCount, int queryPositionStart = 0,
+                                             int segmentLength = 0) {
+        throwUnlessOk(sentinel_hip_dense_softmax_bwd(probabilities, probabilityBatchStride, gradient, gradientBatchStride, batch,
+                                                     keyCount, queryCount, queryPositionStart, windowSize, globalTokenCount,
+                                                     segmentLength, scale, HipFlashAttention::activeStream()));
+    }
+
 private:
+    static void throwUnlessOk(int code) {
+        if (code == SENTINEL_HIP_OK) return;
+        std::string detail = sentinel_hip_last_error();
+        if (detail.empty()) detail = sentinel_hip_strerror(code);
+        if (code == SENTINEL_HIP_RUNTIME) throw std::runtime_error(detail);
+        throw std::invalid_argument(detail);
+    }
     static void rotate(const char* op, HipMatrix& tensor, int headCount, int headDimension, int pairCount,
                        const HipMatrix& cosTable, const HipMatrix& sinTable, int positionOffset, int segmentLength,
                        int inverse) {

@@ -214,6 +214,29 @@ SENTINEL_HIP_API int sentinel_hip_decode_attention_static(const float* query, co
                                          float* out, int q_heads, int kv_heads, int head_dim, int cache_stride, int length,
                                          float scale, int window_size, int global_token_count, void* stream);
 
+/*
+ * Dense (materialising) attention path of the layer: the scores of one (head, pack) are a keys x queries fp32 matrix,
+ * element (key, query) at base[key * query_count + query]; matrix b of a batch starts b * batch_stride elements on.
+ *
+ * sentinel_hip_dense_softmax_fwd, in place: P = softmax over keys of scale * S with forbidden pairs set to -1e9 first.
+ * Replaces the per-head sequence CudaOps::scaleInPlace, applySparseAttentionMaskInPlace, softmaxInto
+ * (Cuda/CudaCausalSelfAttention.cu:272-275; device bodies Cuda/CudaOps.cu:249-309) for a whole batch of heads with one
+ * launch. A pair is allowed when key <= query and (key < global_token_count or window_size <= 0 or
+ * key >= query - window_size + 1), positions being key and query_position_start + query, or, with segment_length > 0,
+ * key % segment_length and query % segment_length of the same segment (CudaOps.cu:257-283).
+ *
+ * sentinel_hip_dense_softmax_bwd, in place over probability_gradient: dS = scale * P * (dP - sum over keys of dP * P),
+ * zero on forbidden pairs. Replaces CudaOps::softmaxBackwardInto, zeroForbiddenScoreGradientsInPlace, scaleInPlace
+ * (Cuda/CudaCausalSelfAttention.cu:455-457; Cuda/CudaOps.cu:311-344).
+ */
+SENTINEL_HIP_API int sentinel_hip_dense_softmax_fwd(float* scores, int batch, long long batch_stride, int key_count,
+                                                    int query_count, int query_position_start, int window_size,
+                                                    int global_token_count, int segment_length, float scale, void* stream);
+SENTINEL_HIP_API int sentinel_hip_dense_softmax_bwd(const float* probabilities, long long probability_batch_stride,
+                                                    float* probability_gradient, long long gradient_batch_stride, int batch,
+                                                    int key_count, int query_count, int query_position_start, int window_size,
+                                                    int global_token_count, int segment_length, float scale, void* stream);
+
 /* Largest head_dim any kernel here accepts (the CUDA path's CudaFlashAttention::maxHeadDimension is 64). */
 SENTINEL_HIP_API int sentinel_hip_flash_max_head_dim(void);
 

@@ -14,7 +14,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libsentinel_hip_attn.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 SOURCES = ["capi.hip", "flash_fp32.hip", "flash_mfma_fwd.hip", "flash_mfma_bwd.hip", "layout_adapter.hip", "decode_attention.hip",
-           "kernel_timing.hip"]
+           "dense_softmax.hip", "kernel_timing.hip"]
 # packed-fp32 instruction selection is switched off for every device translation unit
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]

@@ -509,6 +509,57 @@ extern "C" int sentinel_hip_rope_rotate(float* tensor, int heads, int head_dim, 
     return SENTINEL_HIP_OK;
 }
 
+namespace {
+
+// argument checks shared by the dense path's two softmax entry points; messages follow
+// CudaOps::applySparseAttentionMaskInPlace (Cuda/CudaOps.cu:1262-1267)
+int check_dense(const char* op, const void* a, const void* b, int batch, long long stride_a, long long stride_b, int key_count,
+                int query_count, int query_position_start, int global_token_count, int segment_length, float scale) {
+    if (!a || !b || batch <= 0 || key_count <= 0 || query_count <= 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty scores", op);
+    const long long elements = (long long)key_count * query_count;
+    if (batch > 65535) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s more than 65535 matrices in one call", op);
+    if (batch > 1 && (stride_a < elements || stride_b < elements))
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s batch stride smaller than one matrix", op);
+    if (global_token_count < 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s globalTokenCount must be >= 0", op);
+    if (query_position_start < 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s queryPositionStart must be >= 0", op);
+    if (segment_length < 0) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s segmentLength must be >= 0", op);
+    if (!std::isfinite(scale)) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s scale must be finite", op);
+    if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
+    return SENTINEL_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" int sentinel_hip_dense_softmax_fwd(float* scores, int batch, long long batch_stride, int key_count, int query_count,
+                                              int query_position_start, int window_size, int global_token_count,
+                                              int segment_length, float scale, void* stream_ptr) {
+    const char* op = "sentinel_hip_dense_softmax_fwd";
+    const int rc = check_dense(op, scores, scores, batch, batch_stride, batch_stride, key_count, query_count, query_position_start,
+                               global_token_count, segment_length, scale);
+    if (rc != SENTINEL_HIP_OK) return rc;
+    const hipError_t err = launch_dense_softmax_fwd(scores, batch, batch_stride, key_count, query_count, query_position_start,
+                                                    window_size, global_token_count, segment_length, scale,
+                                                    static_cast<hipStream_t>(stream_ptr));
+    if (err != hipSuccess) return fail_hip("dense softmax launch", err);
+    return SENTINEL_HIP_OK;
+}
+
+extern "C" int sentinel_hip_dense_softmax_bwd(const float* probabilities, long long probability_batch_stride,
+                                              float* probability_gradient, long long gradient_batch_stride, int batch,
+                                              int key_count, int query_count, int query_position_start, int window_size,
+                                              int global_token_count, int segment_length, float scale, void* stream_ptr) {
+    const char* op = "sentinel_hip_dense_softmax_bwd";
+    const int rc = check_dense(op, probabilities, probability_gradient, batch, probability_batch_stride, gradient_batch_stride,
+                               key_count, query_count, query_position_start, global_token_count, segment_length, scale);
+    if (rc != SENTINEL_HIP_OK) return rc;
+    const hipError_t err = launch_dense_softmax_bwd(probabilities, probability_batch_stride, probability_gradient,
+                                                    gradient_batch_stride, batch, key_count, query_count, query_position_start,
+                                                    window_size, global_token_count, segment_length, scale,
+                                                    static_cast<hipStream_t>(stream_ptr));
+    if (err != hipSuccess) return fail_hip("dense softmax backward launch", err);
+    return SENTINEL_HIP_OK;
+}
+
 extern "C" size_t sentinel_hip_decode_workspace_bytes(int q_heads, int head_dim, int length) {
     if (q_heads <= 0 || head_dim <= 0 || length <= 0) return 0;
     return align_up(decode_workspace_bytes(q_heads, head_dim, length));

@@ -93,6 +93,17 @@ hipError_t launch_rope_rotate_f32(float* tensor, int heads, int head_dim, int st
                                   int position_offset, int segment_length, const float* cos, const float* sin, bool inverse,
                                   hipStream_t stream);
 
+// ---- dense (materialising) path of the layer (dense_softmax.hip): keys x queries fp32 score matrices ----
+// in place: P = softmax over keys of (scale * S, forbidden pairs at -1e9); matrix b starts at scores + b * batch_stride
+hipError_t launch_dense_softmax_fwd(float* scores, int batch, long long batch_stride, int key_count, int query_count,
+                                    int query_position_start, int window, int global_tokens, int segment_length, float scale,
+                                    hipStream_t stream);
+// in place over gradient: dS = scale * P * (dP - sum_keys dP * P), zero on forbidden pairs
+hipError_t launch_dense_softmax_bwd(const float* probabilities, long long probability_batch_stride, float* gradient,
+                                    long long gradient_batch_stride, int batch, int key_count, int query_count,
+                                    int query_position_start, int window, int global_tokens, int segment_length, float scale,
+                                    hipStream_t stream);
+
 // ---- optional per-kernel hipEvent timing (kernel_timing.hip) ----
 class KernelTimer {
 public:

@@ -62,6 +62,11 @@ def load_library():
     lib.sentinel_hip_flash_bwd_sparse.restype = i
     lib.sentinel_hip_rope_rotate.argtypes = [vp] + [i] * 7 + [vp, vp, i, i, vp]
     lib.sentinel_hip_rope_rotate.restype = i
+    ll = ctypes.c_longlong
+    lib.sentinel_hip_dense_softmax_fwd.argtypes = [vp, i, ll] + [i] * 6 + [f, vp]
+    lib.sentinel_hip_dense_softmax_fwd.restype = i
+    lib.sentinel_hip_dense_softmax_bwd.argtypes = [vp, ll, vp, ll] + [i] * 7 + [f, vp]
+    lib.sentinel_hip_dense_softmax_bwd.restype = i
     lib.sentinel_hip_decode_workspace_bytes.argtypes = [i] * 3
     lib.sentinel_hip_decode_workspace_bytes.restype = sz
     lib.sentinel_hip_decode_attention.argtypes = [vp] * 4 + [i] * 5 + [f, i, i, vp, sz, vp]
@@ -177,7 +182,44 @@ def _rope_args(rope, head_dimension):
 
 
 class HipOps:
-    """The two rotary-embedding entry points of Sentinel's CudaOps on MI355X (Cuda/CudaOps.hpp:155-159)."""
+    """The rotary-embedding entry points of Sentinel's CudaOps on MI355X (Cuda/CudaOps.hpp:155-159) and the masked
+    column softmax of the layer's dense attention path (Cuda/CudaOps.hpp:144-153)."""
+
+    @staticmethod
+    def _score_batch(scores, what):
+        if not isinstance(scores, torch.Tensor) or scores.dim() not in (2, 3) or scores.numel() == 0:
+            raise ValueError(f"{what} expects a [keys, queries] matrix or a [batch, keys, queries] stack")
+        _require(scores, None, torch.float32, scores.device, what)
+        if not scores.is_cuda:
+            raise ValueError(f"{what} must be on the GPU")
+        batch = 1 if scores.dim() == 2 else int(scores.shape[0])
+        return batch, int(scores.shape[-2]), int(scores.shape[-1])
+
+    @staticmethod
+    def masked_softmax_in_place(scores, scale, window_size=0, global_token_count=0, query_position_start=0,
+                                segment_length=0, *, stream=None):
+        """CudaOps::scaleInPlace + applySparseAttentionMaskInPlace + softmaxInto over keys x queries score matrices
+        (rows are keys), in place, for a whole stack at once."""
+        batch, keys, queries = HipOps._score_batch(scores, "HipOps::maskedSoftmaxInPlace scores")
+        _check(load_library().sentinel_hip_dense_softmax_fwd(_ptr(scores), batch, keys * queries, keys, queries,
+                                                             int(query_position_start), int(window_size),
+                                                             int(global_token_count), int(segment_length), float(scale),
+                                                             _stream_handle(stream)))
+        return scores
+
+    @staticmethod
+    def masked_softmax_backward_in_place(probabilities, probability_gradient, scale, window_size=0, global_token_count=0,
+                                         query_position_start=0, segment_length=0, *, stream=None):
+        """CudaOps::softmaxBackwardInto + zeroForbiddenScoreGradientsInPlace + scaleInPlace: the score gradient is
+        written over probability_gradient."""
+        batch, keys, queries = HipOps._score_batch(probabilities, "HipOps::maskedSoftmaxBackwardInPlace probabilities")
+        _require(probability_gradient, probabilities.shape, torch.float32, probabilities.device,
+                 "HipOps::maskedSoftmaxBackwardInPlace gradient")
+        _check(load_library().sentinel_hip_dense_softmax_bwd(_ptr(probabilities), keys * queries, _ptr(probability_gradient),
+                                                             keys * queries, batch, keys, queries, int(query_position_start),
+                                                             int(window_size), int(global_token_count), int(segment_length),
+                                                             float(scale), _stream_handle(stream)))
+        return probability_gradient
 
     @staticmethod
     def rotary_rotate_in_place(tensor, head_count, head_dimension, pair_count, cos_table, sin_table, position_offset=0,

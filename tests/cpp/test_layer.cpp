@@ -1,6 +1,9 @@
 // GPU test of the C++ attention layer (include/sentinel_hip/HipCausalSelfAttention.hpp) against the CPU oracle's
 // layer (training step and prefill / decode generation), on the shapes of the reference's own device smoke tests (CudaCausalSelfAttention::runFlashParitySmokeDemo:
 // E=64, H=4, T=48; runGqaCudaSmokeDemo: grouped heads) plus packed batches and head_dim 64 / 128 with MFMA arithmetic.
+// With preferFlashAttention = false the same cases run on the dense materialising path, and flash and dense are compared
+// with each other on the shapes of the reference's flash parity runs (main.cpp:640-643: (E, H, T) = (64,4,48), (768,12,128),
+// (768,12,256)). Multi-head cases (kvHeads == heads) run with the stacked QKV weights.
 // Test infrastructure: the oracle is linked here only as the checker.
 #include "../../include/sentinel_hip/HipCausalSelfAttention.hpp"
 #include "../../oracle/sentinel_attention_oracle.h"
@@ -41,7 +44,7 @@ static void expectThrow(const char* what, Fn fn) {
 }
 
 static void runCase(const char* name, int e, int heads, int kvHeads, int d, int T, int packs, int compute, float tol,
-                    int windowSize = 0, int globalTokenCount = 0) {
+                    int windowSize = 0, int globalTokenCount = 0, bool preferFlash = true) {
     const int qRows = heads * d, kvRows = kvHeads * d, cols = packs * T;
     unsigned state = 2024u + static_cast<unsigned>(e + T);
     const float bound = 1.0f / std::sqrt(static_cast<float>(e));
@@ -89,6 +92,9 @@ static void runCase(const char* name, int e, int heads, int kvHeads, int d, int 
 
     HipFlashAttention::computeType() = compute;
     HipCausalSelfAttention layer = HipCausalSelfAttention::createFrom(host);
+    layer.preferFlashAttention = preferFlash;
+    if (layer.usesFusedQkv() != (heads == kvHeads) || layer.qkvWeight.empty() == (heads == kvHeads))
+        throw std::runtime_error("stacked QKV weights must exist exactly for multi-head layers");
     HipMatrix x, g, y, dx, dwq, dwk, dwv, dwo;
     x.upload(hx, e, cols);
     g.upload(hg, e, cols);
@@ -98,15 +104,62 @@ static void runCase(const char* name, int e, int heads, int kvHeads, int d, int 
                 ek = relErr(dwk.download(), wdk), ev = relErr(dwv.download(), wdv), eo = relErr(dwo.download(), wdo);
     std::printf("  %-40s  Y=%.2e dX=%.2e dWq=%.2e dWk=%.2e dWv=%.2e dWo=%.2e\n", name, ey, ex, eq, ek, ev, eo);
     if (ey > tol || ex > tol || eq > tol || ek > tol || ev > tol || eo > tol) throw std::runtime_error(std::string(name) + " parity failed");
-    if (!layer.usedFlashAttention || layer.activePackCount != packs || layer.activeSegmentLength != T)
+    if (layer.usedFlashAttention != preferFlash || layer.activePackCount != packs || layer.activeSegmentLength != T)
         throw std::runtime_error("layer bookkeeping");
+    if (heads == kvHeads) {
+        // the stacked weight gradient alone (materializeSplitWeightGrads = false) holds the same three blocks
+        HipMatrix dx2, a, b, c, o2;
+        layer.backward(g, dx2, a, b, c, o2, false);
+        if (!a.empty() || !b.empty() || !c.empty()) throw std::runtime_error("split weight gradients were materialised");
+        std::vector<float> stacked = layer.qkvWeightGradient.download(), want3(wdq);
+        want3.insert(want3.end(), wdk.begin(), wdk.end());
+        want3.insert(want3.end(), wdv.begin(), wdv.end());
+        if (stacked.size() != want3.size() || relErr(stacked, want3) > tol || relErr(dx2.download(), wdx) > tol)
+            throw std::runtime_error(std::string(name) + " stacked weight gradient parity failed");
+    }
+}
+
+// flash and dense paths of one layer on the same input: outputs and all gradients within tol of each other
+static void runFlashVersusDense(const char* name, int e, int heads, int T, float tol) {
+    const int d = e / heads;
+    unsigned state = 77u + static_cast<unsigned>(e + T);
+    const float bound = 1.0f / std::sqrt(static_cast<float>(e));
+    HostAttentionWeights host;
+    host.queryWeight = lcg(static_cast<size_t>(e) * e, state, bound);
+    host.keyWeight = lcg(static_cast<size_t>(e) * e, state, bound);
+    host.valueWeight = lcg(static_cast<size_t>(e) * e, state, bound);
+    host.outputWeight = lcg(static_cast<size_t>(e) * e, state, bound);
+    host.embeddingDim = e;
+    host.headCount = heads;
+    host.kvHeadCount = heads;
+    host.headDimension = d;
+    host.maximumPositionCount = T;
+    auto hx = lcg(static_cast<size_t>(e) * T, state, 1.0f);
+    auto hg = lcg(static_cast<size_t>(e) * T, state, 1.0f);
+    HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
+    std::vector<std::vector<float>> results[2];
+    for (int pass = 0; pass < 2; ++pass) {
+        HipCausalSelfAttention layer = HipCausalSelfAttention::createFrom(host);
+        layer.preferFlashAttention = pass == 0;
+        HipMatrix x, g, y, dx, dwq, dwk, dwv, dwo;
+        x.upload(hx, e, T);
+        g.upload(hg, e, T);
+        layer.forward(x, y);
+        layer.backward(g, dx, dwq, dwk, dwv, dwo);
+        if (layer.usedFlashAttention != (pass == 0)) throw std::runtime_error("wrong attention path");
+        results[pass] = {y.download(), dx.download(), dwq.download(), dwk.download(), dwv.download(), dwo.download()};
+    }
+    float worst = 0.0f;
+    for (size_t i = 0; i < results[0].size(); ++i) worst = std::max(worst, relErr(results[0][i], results[1][i]));
+    std::printf("  %-40s  flash vs dense worst %.2e\n", name, worst);
+    if (worst > tol) throw std::runtime_error(std::string(name) + " flash / dense parity failed");
 }
 
 // Generation: prefill `prompt` columns, then decode the rest one token at a time. Step t must reproduce column t of
 // the oracle's full forward over columns 0..t (causal attention: earlier columns do not depend on later ones, so
 // one oracle call over all columns gives every step's answer).
 static void runGeneration(const char* name, int e, int heads, int kvHeads, int d, int prompt, int total, int compute, float tol,
-                          int windowSize = 0, int globalTokenCount = 0) {
+                          int windowSize = 0, int globalTokenCount = 0, bool preferFlash = true) {
     const int qRows = heads * d, kvRows = kvHeads * d;
     unsigned state = 4711u + static_cast<unsigned>(e + total);
     const float bound = 1.0f / std::sqrt(static_cast<float>(e));
@@ -132,6 +185,7 @@ static void runGeneration(const char* name, int e, int heads, int kvHeads, int d
 
     HipFlashAttention::computeType() = compute;
     HipCausalSelfAttention layer = HipCausalSelfAttention::createFrom(host);
+    layer.preferFlashAttention = preferFlash;
     HipKvCache cache;
     auto columns = [&](const std::vector<float>& m, int c0, int count) {
         std::vector<float> out(static_cast<size_t>(e) * count);
@@ -180,6 +234,17 @@ int main() {
         runCase("sparse bf16 E256 H4 d64 T300 W70 G10", 256, 4, 4, 64, 300, 1, SENTINEL_HIP_COMPUTE_BF16, 2e-2f, 70, 10);
         runCase("sparse fp16 GQA 4q/1kv d128 T200 W33 packs2", 256, 4, 1, 128, 200, 2, SENTINEL_HIP_COMPUTE_F16, 2e-2f, 33, 0);
         HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
+        // the dense materialising path (flash switched off) against the oracle layer, then against the flash path
+        runCase("dense fp32 E64 H4 d16 T48", 64, 4, 4, 16, 48, 1, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 0, 0, false);
+        runCase("dense fp32 E64 H4 d16 T48 packs4", 64, 4, 4, 16, 48, 4, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 0, 0, false);
+        runCase("dense fp32 GQA 8q/2kv d8 T16 packs3", 64, 8, 2, 8, 16, 3, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 0, 0, false);
+        runCase("dense fp32 E96 H3 d32 T70 packs2", 96, 3, 3, 32, 70, 2, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 0, 0, false);
+        runCase("dense fp32 GQA 4q/1kv d128 T200", 256, 4, 1, 128, 200, 1, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 0, 0, false);
+        runCase("dense sparse fp32 E32 H2 d16 T16 W4 G2", 32, 2, 2, 16, 16, 1, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 4, 2, false);
+        runCase("dense sparse GQA 8q/2kv d8 T90 W17 G3 packs2", 64, 8, 2, 8, 90, 2, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 17, 3, false);
+        runFlashVersusDense("E64 H4 T48", 64, 4, 48, 1e-4f);
+        runFlashVersusDense("E768 H12 T128", 768, 12, 128, 1e-4f);
+        runFlashVersusDense("E768 H12 T256", 768, 12, 256, 1e-4f);
         // the shapes of runKvCacheSmokeDemo (E=64, H=4, T=32 of 64 positions), grouped heads, a cache of several chunks
         runGeneration("generate fp32 E64 H4 d16 32+32", 64, 4, 4, 16, 32, 64, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
         runGeneration("generate fp32 GQA 8q/2kv d8 5+20", 64, 8, 2, 8, 5, 25, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
@@ -187,6 +252,8 @@ int main() {
         runGeneration("generate bf16 prefill GQA 4q/1kv d128", 256, 4, 1, 128, 130, 140, SENTINEL_HIP_COMPUTE_BF16, 2e-2f);
         runGeneration("generate sparse fp32 H4 d16 20+60 W9 G2", 64, 4, 4, 16, 20, 80, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 9, 2);
         runGeneration("generate sparse fp32 GQA d64 3+400 W100 G70", 128, 4, 2, 64, 3, 403, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 100, 70);
+        runGeneration("generate dense prefill H4 d16 32+32", 64, 4, 4, 16, 32, 64, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 0, 0, false);
+        runGeneration("generate dense prefill sparse GQA W9 G2", 64, 4, 2, 16, 20, 60, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 9, 2, false);
         HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
 
         // configurations this layer does not run are refused, not approximated
@@ -200,12 +267,31 @@ int main() {
         host.keyWeight = host.queryWeight;
         host.valueWeight = host.queryWeight;
         host.outputWeight = host.queryWeight;
-        HipCausalSelfAttention noFlash = HipCausalSelfAttention::createFrom(host);
-        noFlash.preferFlashAttention = false;
         HipMatrix x, y;
         x.ensureSize(32, 16);
         x.fill(0.1f);
-        expectThrow("flash disabled needs the dense path", [&] { noFlash.forward(x, y); });
+        {
+            // split weights replaced by matrices of their own are stacked again by syncFusedQkvWeight; the split weights
+            // of a fresh layer are views of the stacked matrix (no copy to keep in step)
+            HipCausalSelfAttention layer = HipCausalSelfAttention::createFrom(host);
+            if (layer.queryWeight.buffer.deviceData != layer.qkvWeight.buffer.deviceData || layer.keyWeight.buffer.ownsMemory)
+                throw std::runtime_error("split weights are not views of the stacked weights");
+            HipMatrix before, after, varied;  // columns that differ, so that the keys matter
+            varied.upload(lcg(32 * 16, st, 1.0f), 32, 16);
+            layer.forward(varied, before);
+            HipMatrix own;
+            own.upload(lcg(32 * 32, st, 0.2f), 32, 32);
+            layer.keyWeight = std::move(own);
+            layer.syncFusedQkvWeight();
+            if (layer.keyWeight.buffer.ownsMemory || layer.keyWeight.buffer.deviceData != layer.qkvWeight.buffer.deviceData + 32 * 32)
+                throw std::runtime_error("syncFusedQkvWeight did not re-stack");
+            layer.forward(varied, after);
+            if (relErr(after.download(), before.download()) < 1e-3f) throw std::runtime_error("new key weights had no effect");
+            layer.releaseActivationScratch();
+            if (!layer.query.empty() || !layer.inputCache.empty() || layer.qkvWeight.empty())
+                throw std::runtime_error("releaseActivationScratch");
+            layer.forward(x, after);
+        }
         HipCausalSelfAttention dense = HipCausalSelfAttention::createFrom(host);
         expectThrow("columns not a multiple of the segment", [&] { dense.forward(x, y, 5); });
         HipMatrix longer;
