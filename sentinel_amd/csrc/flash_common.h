@@ -61,9 +61,14 @@ bool mfma_supported(int head_dim);
 // lse rows are addressed through `lm`; delta is q_heads x (packs * seq_len)
 hipError_t launch_fwd_mfma(Elem type, const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm,
                            AttnGeom g, hipStream_t stream);
+// ds_scratch: bwd_stored_scratch_bytes(g) bytes for the one-pass backward (dS written by the dK / dV kernel, dQ formed
+// from it), or nullptr for the two-pass backward that recomputes S and dP in a dQ kernel of its own
 hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* v, const void* out, const float* lse,
                            RowMap lm, const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g,
-                           hipStream_t stream);
+                           hipStream_t stream, void* ds_scratch = nullptr);
+// 0 where the one-pass backward does not apply (head_dim other than 128, no causal mask, sparse mask, a head's blocks
+// beyond 2 GiB)
+size_t bwd_stored_scratch_bytes(const AttnGeom& g);
 
 // ---- layout adapter (layout_adapter.hip): Sentinel column layout fp32 <-> [B,H,T,d] bf16 / fp16 ----
 // Rotary embedding tables [positions][head_dim / 2] (cos == nullptr: no rotation); token t of a pack uses

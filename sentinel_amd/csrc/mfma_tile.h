@@ -259,7 +259,9 @@ __device__ __forceinline__ void take_priority_turn(unsigned realtime, unsigned t
 // instructions of one wavefront execute in order, so no wait is needed between the writes and the reads.
 // PIN_ADDRESSES keeps the per-lane address arithmetic at the call site: hoisted over the caller's loops it costs about
 // twenty registers there, which the kernels that already use all 256 pay for with spills.
-template <class E, int D, bool PIN_ADDRESSES = true, int ROWS_PER_PASS = 32>
+// OPERAND_ORDER: block row r is not matrix row r but, inside its group of 16, row 2 (r / 8) + rho(r % 8), the order in
+// which a B operand holds contraction indices (see the header comment).
+template <class E, int D, bool PIN_ADDRESSES = true, int ROWS_PER_PASS = 32, bool OPERAND_ORDER = false>
 __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], float factor, unsigned short* lds,
                                                    unsigned short* dst, int valid_rows, int lane) {
     constexpr int PIECES = D / 8;          // 16-byte pieces per row
@@ -291,7 +293,8 @@ __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], 
         for (int i = 0; i < ROWS_PER_PASS / ROWS_PER_STORE; ++i) {
             const int r = i * ROWS_PER_STORE + lane / PIECES;
             const u32x4 val = *reinterpret_cast<const u32x4*>(base + r * (D * 2) + ((p ^ (r & (PIECES - 1))) << 4));
-            const int out_row = pass * ROWS_PER_PASS + r;
+            int out_row = pass * ROWS_PER_PASS + r;
+            if (OPERAND_ORDER) out_row = (out_row & ~15) | (((out_row >> 3) & 1) << 1) | ((out_row & 3) << 2) | ((out_row >> 2) & 1);
             if (out_row < valid_rows) *reinterpret_cast<u32x4*>(dst + (long long)out_row * D + p * 8) = val;
         }
         __builtin_amdgcn_wave_barrier();

@@ -42,11 +42,11 @@ def _inputs(name):
     return q, k, v, g
 
 
-def _run(q, k, v, g):
+def _run(q, k, v, g, **backward_options):
     from sentinel_amd import flash_attention_backward, flash_attention_forward
     out, lse = flash_attention_forward(q, k, v)
     dq, dk, dv = (torch.full_like(x, float("nan")) for x in (q, k, v))
-    flash_attention_backward(q, k, v, out, lse, g, dq=dq, dk=dk, dv=dv)
+    flash_attention_backward(q, k, v, out, lse, g, dq=dq, dk=dk, dv=dv, **backward_options)
     torch.cuda.synchronize()
     return out, lse, dq, dk, dv
 
@@ -85,6 +85,19 @@ def test_slice_matches_oracle_at_full_length(name, where):
     out, lse, dq, dk, dv = _run(q, k, v, g)
     _check_slice(name, where, out, lse, dq, dk, dv, q, k, v, g)
     for x in (out, lse, dq, dk, dv):
+        assert torch.isfinite(x.float()).all(), "non-finite value outside the checked slice"
+
+
+@pytest.mark.parametrize("where", ["first", "last"])
+@pytest.mark.parametrize("name", ["c4_gqa", "target_shape"])
+def test_stored_scores_backward_at_full_length(name, where):
+    """The one-pass backward variant (dS written by the dK / dV kernel, dQ formed from it; 2 GiB of scores at these shapes)
+    at the full size: the two ends of the grids' walk against the oracle."""
+    print(f"case {name} {where} stored-scores backward vs oracle", flush=True)
+    q, k, v, g = _inputs(name)
+    out, lse, dq, dk, dv = _run(q, k, v, g, stored_scores=True)
+    _check_slice(name, where, out, lse, dq, dk, dv, q, k, v, g)
+    for x in (dq, dk, dv):
         assert torch.isfinite(x.float()).all(), "non-finite value outside the checked slice"
 
 
