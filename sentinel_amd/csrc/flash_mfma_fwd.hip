@@ -65,14 +65,16 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     // query tiles (launching a workgroup costs about 5 us of its slot, a sixth of an average tile at T = 4096).
     // Workgroup ids are dealt round-robin to the 8 XCDs; each XCD owns a contiguous range of tiles (head-major,
     // longest query tile of a head first), so the query tiles of one head, which stream the same K / V, share one
-    // L2.  Round r hands the XCD's tiles [r S, (r + 1) S) to its S workgroups, forwards in even rounds and backwards
-    // in odd ones: long and short tiles alternate and every workgroup ends up with about the same work.
+    // L2.  query_tile_of_slot hands them out so that every workgroup, and every compute unit, ends up with about
+    // the same work.
     const unsigned turn_class = priority_turn_class();
     const int xcd = (int)blockIdx.x % kXcds;
     const int slot = (int)blockIdx.x / kXcds;
     const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
-    const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
+    // (under the sparse mask one workgroup per tile is launched, more than run at once, and tile lengths do not follow
+    //  the tile index: plain order)
+    const int local_tile = WINDOW ? round * slots + slot : query_tile_of_slot(slot, slots, round, tiles_per_xcd, q_tiles);
     const int tile_id = xcd * tiles_per_xcd + local_tile;
     if (local_tile >= tiles_per_xcd || tile_id >= total_tiles) break;
     const int bh = tile_id / q_tiles;

@@ -305,6 +305,29 @@ __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], 
 // round-robin to them, so workgroup id % kXcds names the die a workgroup runs on.
 constexpr int kXcds = 8;
 
+// Which tile of its XCD a workgroup of a query-outer persistent grid takes in `round`.  The XCD's tiles are numbered
+// head-major, the longest (last) query tile of a head first; `slot` = workgroup id / kXcds of `slots`.
+// * Several rounds: round r hands tiles [r S, (r + 1) S) to the S workgroups, forwards in even rounds and backwards in
+//   odd ones, so long and short tiles alternate for every workgroup and the tiles of a head stay neighbours (they share
+//   that head's K / V in the XCD's L2).
+// * One round only (a small problem: every tile has a workgroup of its own): the hardware places workgroups s, s + 32,
+//   s + 64 .. of an XCD on the same compute unit (32 per XCD), and with head-major numbering those are tiles of the same
+//   length whenever the tiles per head divide 32: one compute unit would get only the longest tiles, another only the
+//   shortest (a factor of 8 at 8 tiles per head).  The tiles are then taken length-major (all longest first) and dealt
+//   to the compute units in snake order, so that the workgroups sharing a compute unit hold long and short ones.
+// Returns the head-major tile index inside the XCD.
+constexpr int kCusPerXcd = 32;
+__device__ __forceinline__ int query_tile_of_slot(int slot, int slots, int round, int tiles_per_xcd, int q_tiles) {
+    if (slots >= tiles_per_xcd && slots % kCusPerXcd == 0 && tiles_per_xcd % q_tiles == 0) {
+        if (round > 0) return tiles_per_xcd;  // nothing left
+        const int pass = slot / kCusPerXcd, cu = slot % kCusPerXcd;
+        const int sorted = pass * kCusPerXcd + ((pass & 1) ? kCusPerXcd - 1 - cu : cu);  // position in length-major order
+        const int heads = tiles_per_xcd / q_tiles;
+        return sorted < tiles_per_xcd ? (sorted % heads) * q_tiles + sorted / heads : tiles_per_xcd;
+    }
+    return round * slots + ((round & 1) ? slots - 1 - slot : slot);
+}
+
 // Workgroups the device runs at once, per XCD: occupancy of the kernel times the compute units of an XCD.
 template <typename Kernel>
 inline int resident_workgroups_per_xcd(Kernel kernel, int threads, size_t dynamic_lds) {
