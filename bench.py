@@ -35,8 +35,8 @@ SEEDS = {"c1": 1, "c2": 2, "c3": 3, "c4": 4, "c5": 5, "nstar": 6}
 # algorithmic matrix products per kernel (units of B*H*T^2*d FLOPs, causal-halved)
 KERNEL_UNITS = {"fwd_mfma": 2.0, "dkdv_mfma": 4.0, "dq_mfma": 1.0, "fwd_f32": 2.0, "dkdv_f32": 4.0, "dq_f32": 1.0}
 # kernel names as timed by the library -> the kernel functions they stand for in the profiler's tables
-PROFILED_KERNELS = {"fwd_mfma": ("fwd_mfma_kernel", "fwd_pingpong_kernel"), "dkdv_mfma": ("dkdv_split_kernel", "dkdv_mfma_kernel"),
-                    "dq_mfma": ("dq_mfma_kernel", "dq_pingpong_kernel")}
+PROFILED_KERNELS = {"fwd_mfma": ("fwd_mfma_kernel",), "dkdv_mfma": ("dkdv_split_kernel", "dkdv_mfma_kernel"),
+                    "dq_mfma": ("dq_mfma_kernel",)}
 COUNTER_SUMMARIES = {"nstar": "nstar_b4_h32_t4096_d128_bf16_counters.txt"}
 
 

@@ -73,8 +73,11 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
     // (under the sparse mask one workgroup per tile is launched, more than run at once, and tile lengths do not follow
-    //  the tile index: plain order)
-    const int local_tile = WINDOW ? round * slots + slot : query_tile_of_slot(slot, slots, round, tiles_per_xcd, q_tiles);
+    //  the tile index: plain order.  At head_dim 128 the kernel has no register to spare for the one-round case of
+    //  query_tile_of_slot: it costs two spilled registers there, so only the snake over rounds is used.)
+    const int local_tile = WINDOW   ? round * slots + slot
+                           : D > 64 ? round * slots + ((round & 1) ? slots - 1 - slot : slot)
+                                    : query_tile_of_slot(slot, slots, round, tiles_per_xcd, q_tiles);
     const int tile_id = xcd * tiles_per_xcd + local_tile;
     if (local_tile >= tiles_per_xcd || tile_id >= total_tiles) break;
     const int bh = tile_id / q_tiles;

@@ -322,8 +322,18 @@ __device__ __forceinline__ int query_tile_of_slot(int slot, int slots, int round
         if (round > 0) return tiles_per_xcd;  // nothing left
         const int pass = slot / kCusPerXcd, cu = slot % kCusPerXcd;
         const int sorted = pass * kCusPerXcd + ((pass & 1) ? kCusPerXcd - 1 - cu : cu);  // position in length-major order
-        const int heads = tiles_per_xcd / q_tiles;
-        return sorted < tiles_per_xcd ? (sorted % heads) * q_tiles + sorted / heads : tiles_per_xcd;
+        if (sorted >= tiles_per_xcd) return tiles_per_xcd;
+        // position `sorted` of the length-major order = tile `rank` (0: longest) of head sorted - rank * heads; a scalar
+        // loop over the few tiles of a head instead of two divisions by run-time values (whose temporaries cost the
+        // 256-register kernels a spill)
+        int heads = 0;
+        for (int t = 0; t < tiles_per_xcd; t += q_tiles) ++heads;
+        int rank = 0, first = 0;
+        while (first + heads <= sorted) {
+            first += heads;
+            ++rank;
+        }
+        return (sorted - first) * q_tiles + rank;
     }
     return round * slots + ((round & 1) ? slots - 1 - slot : slot);
 }
