@@ -51,7 +51,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                                                                   const float* __restrict__ lse,
                                                                   float* __restrict__ delta,
                                                                   unsigned short* __restrict__ dq, RowMap lm, AttnGeom g,
-                                                                  int q_tiles, int total_tiles, int tiles_per_xcd) {
+                                                                  int q_tiles, int total_tiles, int tiles_per_xcd, int deal) {
     constexpr int KT = kDqKeyTile;
     typedef DirectTile<KT, D, kBwdThreads> Tile;
     constexpr int KSTEPS = D / 16;
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
     const int slot = (int)blockIdx.x / kXcds;
     const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
-    const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
+    const int local_tile = tile_of_slot(slot, slots, round, tiles_per_xcd, q_tiles, deal);
     const int tile_id = xcd * tiles_per_xcd + local_tile;
     if (local_tile >= tiles_per_xcd || tile_id >= total_tiles) break;
     const int bh = tile_id / q_tiles;
@@ -668,7 +668,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
-    int total_tiles, int tiles_per_xcd) {
+    int total_tiles, int tiles_per_xcd, int deal) {
     constexpr int QT = kDkvQueryTile;
     typedef RowTile<QT, D, kBwdThreads, DkvLds<D>::kPad> RTile;
     constexpr int QS = RTile::kStride;
@@ -694,7 +694,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     const int slot = (int)blockIdx.x / kXcds;
     const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
-    const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
+    const int local_tile = tile_of_slot(slot, slots, round, tiles_per_xcd, k_tiles, deal);
     int bkv, ktile;
     if (local_tile >= tiles_per_xcd ||
         !dkv_tile_of_workgroup(xcd, local_tile, tiles_per_xcd, k_tiles, total_tiles, front_tiles, bkv, ktile))
@@ -902,7 +902,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
-    int total_tiles, int tiles_per_xcd, unsigned short* __restrict__ ds_out) {
+    int total_tiles, int tiles_per_xcd, int deal, unsigned short* __restrict__ ds_out) {
     static_assert(!(STORE_DS && WINDOW), "the stored score gradients cover the full causal / full rectangle only");
     constexpr int QT = kDkvQueryTile;
     // the query / dO tiles of a stage are staged by the score wavefronts alone (threads 0..255): they have about a
@@ -932,7 +932,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const int slot = (int)blockIdx.x / kXcds;
     const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
-    const int local_tile = round * slots + ((round & 1) ? slots - 1 - slot : slot);
+    const int local_tile = tile_of_slot(slot, slots, round, tiles_per_xcd, k_tiles, deal);
     int bkv, ktile;
     if (local_tile >= tiles_per_xcd ||
         !dkv_tile_of_workgroup(xcd, local_tile, tiles_per_xcd, k_tiles, total_tiles, front_tiles, bkv, ktile))
@@ -1306,7 +1306,7 @@ hipError_t run_bwd_stored(const unsigned short* qp, const unsigned short* kp, co
             const int grid = kXcds * (tiles_per_xcd < resident ? tiles_per_xcd : resident);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp, dvp, lm, g,
-                               k_tiles, total, tiles_per_xcd, ds);
+                               k_tiles, total, tiles_per_xcd, 0, ds);
             return hipGetLastError();
         };
         const hipError_t err = launch(dkdv_split_kernel<E, D, true, false, true>);
@@ -1349,14 +1349,16 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
         const int q_tiles = (T + kDqQueryTile - 1) / kDqQueryTile;
         const int total = g.packs * g.q_heads * q_tiles;
         const int tiles_per_xcd = (total + kXcds - 1) / kXcds;
+        const long long streamed = 2ll * T * D * 2;  // K and V of a head
         auto launch = [&](auto kernel) {
             static const int resident = resident_workgroups_per_xcd(kernel, kBwdThreads, 0);  // per kernel instantiation
             // under the sparse mask tile lengths no longer grow with the tile index, and one workgroup per tile handed out
             // as slots free up is 6 - 13 % faster than the fixed snake assignment
-            const int grid = kXcds * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
+                                               : plan_persistent_grid(tiles_per_xcd, q_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dq_mfma", stream);
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp, lse, delta, dqp, lm, g,
-                               q_tiles, total, tiles_per_xcd);
+            hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp, lse, delta, dqp,
+                               lm, g, q_tiles, total, tiles_per_xcd, plan.deal);
         };
         if (g.window > 0)
             launch(dq_mfma_kernel<E, D, true, true>);
@@ -1371,16 +1373,18 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
     const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
     const int total = g.packs * g.kv_heads * k_tiles;
     const int tiles_per_xcd = (total + kXcds - 1) / kXcds;
+    const long long streamed = 2ll * (g.q_heads / g.kv_heads) * T * D * 2;  // Q and dO of the heads that share a K / V head
     if constexpr (D <= 64) {
         const size_t smem = 2 * sizeof(DkvLds<D>);
         auto launch = [&](auto kernel) {
             static const int resident = resident_workgroups_per_xcd(kernel, kBwdThreads, smem);  // per kernel instantiation
             // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
             // dispatched in order (long ones first), balances better than a fixed assignment
-            const int grid = kXcds * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
+                                               : plan_persistent_grid(tiles_per_xcd, k_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dkdv_mfma", stream);
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp, dvp, lm, g,
-                               k_tiles, total, tiles_per_xcd);
+            hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp,
+                               dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal);
         };
         if (g.window > 0)
             launch(dkdv_mfma_kernel<E, D, true, true>);
@@ -1399,10 +1403,11 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
             static const int resident = resident_workgroups_per_xcd(kernel, kDkvSplitThreads, smem);
             // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
             // dispatched in order (long ones first), balances better than a fixed assignment
-            const int grid = kXcds * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+            const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
+                                               : plan_persistent_grid(tiles_per_xcd, k_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dkdv_mfma", stream);
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp, dvp, lm, g,
-                               k_tiles, total, tiles_per_xcd, static_cast<unsigned short*>(nullptr));
+            hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp,
+                               dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal, static_cast<unsigned short*>(nullptr));
             return hipGetLastError();
         };
         if (g.window > 0)

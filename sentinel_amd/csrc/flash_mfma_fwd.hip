@@ -40,7 +40,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
                                                                    const unsigned short* __restrict__ v,
                                                                    unsigned short* __restrict__ out,
                                                                    float* __restrict__ lse, RowMap lm, AttnGeom g,
-                                                                   int q_tiles, int total_tiles, int tiles_per_xcd) {
+                                                                   int q_tiles, int total_tiles, int tiles_per_xcd, int deal) {
     constexpr int KT = kFwdKeyTile;
     typedef DirectTile<KT, D, kFwdThreads> Tile;
     constexpr int KSTEPS = D / 16;  // k-steps of the S^T product
@@ -73,11 +73,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     const int slots = (int)gridDim.x / kXcds;
     for (int round = 0;; ++round) {
     // (under the sparse mask one workgroup per tile is launched, more than run at once, and tile lengths do not follow
-    //  the tile index: plain order.  At head_dim 128 the kernel has no register to spare for the one-round case of
-    //  query_tile_of_slot: it costs two spilled registers there, so only the snake over rounds is used.)
-    const int local_tile = WINDOW   ? round * slots + slot
-                           : D > 64 ? round * slots + ((round & 1) ? slots - 1 - slot : slot)
-                                    : query_tile_of_slot(slot, slots, round, tiles_per_xcd, q_tiles);
+    //  the tile index: plain order)
+    const int local_tile = WINDOW ? round * slots + slot
+                                  : __builtin_amdgcn_readfirstlane(tile_of_slot(slot, slots, round, tiles_per_xcd, q_tiles, deal));
     const int tile_id = xcd * tiles_per_xcd + local_tile;
     if (local_tile >= tiles_per_xcd || tile_id >= total_tiles) break;
     const int bh = tile_id / q_tiles;
@@ -289,6 +287,7 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
     const int q_tiles = (g.seq_len + kFwdQueryTile - 1) / kFwdQueryTile;
     const int total = g.packs * g.q_heads * q_tiles;
     const int tiles_per_xcd = (total + kXcds - 1) / kXcds;
+    const long long streamed = 2ll * g.seq_len * D * 2;  // K and V of a head
     auto qp = static_cast<const unsigned short*>(q);
     auto kp = static_cast<const unsigned short*>(k);
     auto vp = static_cast<const unsigned short*>(v);
@@ -297,10 +296,11 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
         static const int resident = resident_workgroups_per_xcd(kernel, kFwdThreads, 0);  // per kernel instantiation
         // under the sparse mask tile lengths no longer grow with the tile index, and one workgroup per tile handed out
         // as slots free up is 6 - 13 % faster than the fixed snake assignment
-        const int grid = kXcds * (g.window > 0 || tiles_per_xcd < resident ? tiles_per_xcd : resident);
+        const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
+                                           : plan_persistent_grid(tiles_per_xcd, q_tiles, resident, g.causal != 0, streamed);
         KernelTimer timer("fwd_mfma", stream);
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm, g, q_tiles, total,
-                           tiles_per_xcd);
+        hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm, g, q_tiles,
+                           total, tiles_per_xcd, plan.deal);
     };
     if (g.window > 0)
         launch(fwd_mfma_kernel<E, D, true, true>);
