@@ -30,6 +30,7 @@ constexpr int kFwdQueryTile = 128;
 // instruction classes of __builtin_amdgcn_sched_group_barrier
 constexpr int kSchedMfma = 0x008;
 constexpr int kSchedDsRead = 0x100;
+constexpr int kSchedVmem = 0x010;
 constexpr int kOperandLead = 4;
 
 constexpr int kFwdKeyTile = 64;
@@ -140,10 +141,15 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     // one trip over the tile held in (k_cur, v_cur); the next tile streams into (k_next, v_next) meanwhile
     auto tile_trip = [&](int j, const unsigned short* k_cur, const unsigned short* v_cur, unsigned short* k_next,
                          unsigned short* v_next) __attribute__((always_inline)) {
-        const bool more = j + 1 < n_trips;
-        if (more) {
-            Tile::issue(k_rsrc, k_next, ld_off, tile_of(j + 1) * KT * D * 2, wave);
-            Tile::issue(v_rsrc, v_next, ld_off, tile_of(j + 1) * KT * D * 2, wave);
+        // the next tile's requests go out between the matrix instructions of the score chains (a wavefront is held for
+        // 40 - 60 cycles per request, which then passes while its own matrix instructions run); the last trip fetches
+        // its own tile once more, which nobody reads
+        const int next_bytes = tile_of(j + 1 < n_trips ? j + 1 : j) * KT * D * 2;
+        // (under the sparse mask a wavefront may skip trips in mid-tile; there the requests go out first, as a block)
+        constexpr bool SPREAD = !WINDOW;
+        if (!SPREAD && j + 1 < n_trips) {
+            Tile::issue(k_rsrc, k_next, ld_off, next_bytes, wave);
+            Tile::issue(v_rsrc, v_next, ld_off, next_bytes, wave);
         }
 
         const int key0 = tile_of(j) * KT;
@@ -168,22 +174,29 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) s[kbk] = E::mfma(kfrag[kbk][ks], qf[ks], s[kbk]);
             }
+            if (SPREAD) {
+                Tile::issue(k_rsrc, k_next, ld_off, next_bytes, wave);
+                Tile::issue(v_rsrc, v_next, ld_off, next_bytes, wave);
+            }
 #pragma unroll
             for (int c4 = 0; c4 < 2; ++c4)
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
                     vfrag[c4][cb] = lds_read_transposed_pair(v_cur + c4 * 16 * D + (t_even ^ (cb << 5)),
                                                              v_cur + c4 * 16 * D + (t_odd ^ (cb << 5)));
+            static_assert(2 * Tile::kIters == KSTEPS, "one request per two matrix instructions of the score chains");
             __builtin_amdgcn_sched_group_barrier(kSchedDsRead, kOperandLead, 0);
 #pragma unroll
             for (int i = 0; i < 2 * KSTEPS - kOperandLead; ++i) {
                 __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 1, 0);
+                if (SPREAD && (i & 1)) __builtin_amdgcn_sched_group_barrier(kSchedVmem, 1, 0);
             }
 #pragma unroll
             for (int i = 0; i < kOperandLead; ++i) {
                 __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(kSchedDsRead, 4 * CB / kOperandLead, 0);
+                if (SPREAD && (i & 1)) __builtin_amdgcn_sched_group_barrier(kSchedVmem, 1, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
 
@@ -256,7 +269,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
             }
             __builtin_amdgcn_sched_group_barrier(kSchedMfma, 2 * CB, 0);
             __builtin_amdgcn_sched_barrier(0);
-        }
+        }  // (under the plain causal mask a wavefront skips only the last trip of its tile, after which nothing is read)
 
         // priority turns: for the persistent grid with two workgroups per compute unit (head_dim 128) only
         constexpr bool TURNS = !WINDOW && D > 64;
