@@ -1355,7 +1355,7 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
             // under the sparse mask tile lengths no longer grow with the tile index, and one workgroup per tile handed out
             // as slots free up is 6 - 13 % faster than the fixed snake assignment
             const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
-                                               : plan_persistent_grid(tiles_per_xcd, q_tiles, resident, g.causal != 0, streamed);
+                                               : plan_persistent_grid(total, q_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dq_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp, lse, delta, dqp,
                                lm, g, q_tiles, total, tiles_per_xcd, plan.deal);
@@ -1381,7 +1381,7 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
             // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
             // dispatched in order (long ones first), balances better than a fixed assignment
             const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
-                                               : plan_persistent_grid(tiles_per_xcd, k_tiles, resident, g.causal != 0, streamed);
+                                               : plan_persistent_grid(total, k_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp,
                                dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal);
@@ -1404,7 +1404,7 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
             // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
             // dispatched in order (long ones first), balances better than a fixed assignment
             const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
-                                               : plan_persistent_grid(tiles_per_xcd, k_tiles, resident, g.causal != 0, streamed);
+                                               : plan_persistent_grid(total, k_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp,
                                dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal, static_cast<unsigned short*>(nullptr));

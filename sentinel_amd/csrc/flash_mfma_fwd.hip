@@ -310,7 +310,7 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
         // under the sparse mask tile lengths no longer grow with the tile index, and one workgroup per tile handed out
         // as slots free up is 6 - 13 % faster than the fixed snake assignment
         const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
-                                           : plan_persistent_grid(tiles_per_xcd, q_tiles, resident, g.causal != 0, streamed);
+                                           : plan_persistent_grid(total, q_tiles, resident, g.causal != 0, streamed);
         KernelTimer timer("fwd_mfma", stream);
         hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm, g, q_tiles,
                            total, tiles_per_xcd, plan.deal);

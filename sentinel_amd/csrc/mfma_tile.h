@@ -355,7 +355,7 @@ inline int resident_workgroups_per_xcd(Kernel kernel, int threads, size_t dynami
     return per_cu * ((cus + kXcds - 1) / kXcds);
 }
 
-// Grid of a persistent kernel over `tiles_per_xcd` tiles per XCD, `tiles_per_head` of them per head, `resident` workgroups
+// Grid of a persistent kernel over `total_tiles` tiles (an eighth per XCD, rounded up), `tiles_per_head` of them per head, `resident` workgroups
 // running at once per XCD; `streamed_bytes_per_head` = the operands every tile of a head streams (K and V, or Q and dO).
 // Chooses between the head-major snake and the length-major deal of tile_of_slot:
 // * the deal gives up the reuse of a head's streamed operands between neighbouring workgroups, so it is considered only
@@ -380,11 +380,16 @@ inline long long busiest_compute_unit(int slots, int tiles_per_xcd, int tiles_pe
     for (long long l : load) most = l > most ? l : most;
     return most;
 }
-inline GridPlan plan_persistent_grid(int tiles_per_xcd, int tiles_per_head, int resident, bool lengths_differ,
+inline GridPlan plan_persistent_grid(int total_tiles, int tiles_per_head, int resident, bool lengths_differ,
                                      long long streamed_bytes_per_head) {
     constexpr long long kDealFootprintLimit = 8ll << 20;
+    const int tiles_per_xcd = (total_tiles + kXcds - 1) / kXcds;
     const GridPlan snake{tiles_per_xcd < resident ? tiles_per_xcd : resident, 0};
-    if (!lengths_differ || resident % kCusPerXcd != 0 || tiles_per_xcd % tiles_per_head != 0) return snake;
+    // (every XCD must hold the same whole number of heads: the kernels leave their loop at the first tile past the end
+    //  of the problem, and only the snake meets those last)
+    if (!lengths_differ || resident % kCusPerXcd != 0 || tiles_per_xcd % tiles_per_head != 0 ||
+        total_tiles != kXcds * tiles_per_xcd)
+        return snake;
     if (tiles_per_xcd / tiles_per_head * streamed_bytes_per_head > kDealFootprintLimit) return snake;
     const int passes = (tiles_per_xcd + kCusPerXcd - 1) / kCusPerXcd * kCusPerXcd;
     const GridPlan dealt{passes < resident ? passes : resident, 1};
