@@ -27,6 +27,12 @@ CONFIGS = {
     "c4_gqa": (4, 32, 8, 4096, 128, "bf16", 1.0),
     "c5_long_fp16": (1, 16, 16, 16384, 64, "fp16", 3.0),
     "target_shape": (4, 32, 32, 4096, 128, "bf16", 1.0),
+    # shapes whose persistent grids take the length-major deal of tiles (mfma_tile.h: plan_persistent_grid) in ways the
+    # baseline configurations do not: key tiles dealt over three rounds; query tiles over 2.67 rounds (as C5, in bf16
+    # with more heads per XCD); head_dim 128 query tiles dealt in one round
+    "dealt_keys_d64_t2048": (8, 12, 12, 2048, 64, "bf16", 1.0),
+    "dealt_queries_d64_t4096": (4, 16, 16, 4096, 64, "bf16", 1.0),
+    "dealt_queries_d128_t2048": (1, 32, 32, 2048, 128, "bf16", 1.0),
 }
 
 
