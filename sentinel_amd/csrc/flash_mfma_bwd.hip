@@ -72,8 +72,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 
     // Persistent workgroups: as many as the device runs at once, each walking several query tiles.  Each XCD owns a
     // contiguous range of tiles (head-major, longest query tile of a head first: the tiles of one head stream the same
-    // K / V through one L2); round r hands the XCD's tiles [r S, (r + 1) S) to its S workgroups, forwards in even
-    // rounds and backwards in odd ones, so long and short tiles alternate.
+    // K / V through one L2); tile_of_slot hands them out in the order the host chose (plan_persistent_grid): by default
+    // round r hands the XCD's tiles [r S, (r + 1) S) to its S workgroups, forwards in even rounds and backwards in odd
+    // ones, so long and short tiles alternate.
     const unsigned turn_class = priority_turn_class();
     const int xcd = (int)blockIdx.x % kXcds;
     const int slot = (int)blockIdx.x / kXcds;
@@ -687,7 +688,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     const int n = lane % 32;
     const int gh = lane / 32;
 
-    // persistent workgroups walking the XCD's key tiles in snake order (see dq_mfma_kernel)
+    // persistent workgroups walking the XCD's key tiles in the order the host chose (tile_of_slot; see dq_mfma_kernel)
     const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
     const unsigned turn_class = priority_turn_class();
     const int xcd = (int)blockIdx.x % kXcds;
@@ -926,7 +927,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const int n = lane % 32;
     const int gh = lane / 32;
 
-    // persistent workgroups walking the XCD's key tiles in snake order (see dq_mfma_kernel)
+    // persistent workgroups walking the XCD's key tiles in the order the host chose (tile_of_slot; see dq_mfma_kernel)
     const int front_tiles = WINDOW ? min(k_tiles - 1, (g.global_tokens + kDkvKeyTile - 1) / kDkvKeyTile) : 0;
     const int xcd = (int)blockIdx.x % kXcds;
     const int slot = (int)blockIdx.x / kXcds;

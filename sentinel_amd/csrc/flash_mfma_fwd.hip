@@ -66,8 +66,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     // query tiles (launching a workgroup costs about 5 us of its slot, a sixth of an average tile at T = 4096).
     // Workgroup ids are dealt round-robin to the 8 XCDs; each XCD owns a contiguous range of tiles (head-major,
     // longest query tile of a head first), so the query tiles of one head, which stream the same K / V, share one
-    // L2.  query_tile_of_slot hands them out so that every workgroup, and every compute unit, ends up with about
-    // the same work.
+    // L2.  tile_of_slot hands them out in the order the host chose (plan_persistent_grid), so that every workgroup and
+    // every compute unit ends up with about the same work.
     const unsigned turn_class = priority_turn_class();
     const int xcd = (int)blockIdx.x % kXcds;
     const int slot = (int)blockIdx.x / kXcds;
