@@ -147,6 +147,10 @@ size_t conversion_bytes(const Resolved& r, bool backward) {
     return backward ? 4 * nq + 4 * nkv : 2 * nq + 2 * nkv;
 }
 size_t stored_scores_bytes(const Resolved& r) { return r.stored_scores ? align_up(bwd_stored_scratch_bytes(r.g)) : 0; }
+// The kernels write fp32 column matrices with 32-bit byte offsets inside a head's rows: head_dim rows must span less
+// than 2 GiB (and likewise the rotary tables, which resolve_rope has bounded).
+bool direct_columns(const Resolved& r) { return (long long)r.g.head_dim * r.stride * 4 < 0x7fffffffLL; }
+
 size_t workspace_need(const Resolved& r, bool backward) {
     return conversion_bytes(r, backward) + (backward ? stored_scores_bytes(r) : 0);
 }
@@ -317,8 +321,13 @@ int flash_fwd(const char* op, const void* q, const void* k, const void* v, void*
     if (err == hipSuccess)
         err = launch_columns_to_bhtd(type, static_cast<const float*>(v) + off, v16, g.kv_heads, g.head_dim, stride,
                                      g.seq_len, g.packs, none, stream);
-    if (err == hipSuccess) err = launch_fwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g, stream);
+    // O goes to the caller's matrix straight from the kernel's accumulators (and in 16 bit to the workspace, for the
+    // backward); a conversion pass only where the kernel's 32-bit row offsets would not reach
+    const bool direct = direct_columns(r);
     if (err == hipSuccess)
+        err = launch_fwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g, stream,
+                              direct ? ColumnSink{static_cast<float*>(out) + off, r.stride, none} : kNoColumnSink);
+    if (err == hipSuccess && !direct)
         err = launch_bhtd_to_columns(type, o16, static_cast<float*>(out) + off, g.q_heads, g.head_dim, stride, g.seq_len,
                                      g.packs, none, stream);
     if (err != hipSuccess) return fail_hip("MFMA forward (column layout) launch", err);
@@ -410,10 +419,21 @@ int flash_bwd(const char* op, const void* q, const void* k, const void* v, const
     if (err == hipSuccess)
         err = launch_columns_to_bhtd(type, static_cast<const float*>(d_out) + off, g16, g.q_heads, g.head_dim, stride, T,
                                      g.packs, none, stream);
+    // The gradients leave the kernels as fp32 columns, straight from the accumulators, rotated back on the way (they are
+    // gradients with respect to the unrotated Q, K).  The one-pass variant and matrices beyond the kernels' 32-bit row
+    // offsets write 16-bit tensors and convert them in passes of their own.
+    void* scores = stored_scores_bytes(r) ? ws + conversion_bytes(r, true) : nullptr;
+    if (!scores && direct_columns(r)) {
+        if (err == hipSuccess)
+            err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream, nullptr,
+                                  ColumnSink{static_cast<float*>(dq) + off, r.stride, rope},
+                                  ColumnSink{static_cast<float*>(dk) + off, r.stride, rope},
+                                  ColumnSink{static_cast<float*>(dv) + off, r.stride, none});
+        if (err != hipSuccess) return fail_hip("MFMA backward (column layout) launch", err);
+        return SENTINEL_HIP_OK;
+    }
     if (err == hipSuccess)
-        err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream,
-                              stored_scores_bytes(r) ? ws + conversion_bytes(r, true) : nullptr);
-    // gradients with respect to the unrotated Q, K: the inverse rotation rides on the way out
+        err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream, scores);
     if (err == hipSuccess)
         err = launch_bhtd_to_columns(type, dq16, static_cast<float*>(dq) + off, g.q_heads, g.head_dim, stride, T, g.packs,
                                      rope, stream);

@@ -56,21 +56,6 @@ hipError_t launch_bwd_f32(const float* q, const float* k, const float* v, const 
                           const float* d_out, float* dq, float* dk, float* dv, float* delta, TensorMap qm, TensorMap kvm,
                           RowMap lm, AttnGeom g, hipStream_t stream);
 
-// ---- MFMA path (flash_mfma_*.hip): bf16 / fp16 [B,H,T,d] tensors, head_dim 64 or 128 ----
-bool mfma_supported(int head_dim);
-// lse rows are addressed through `lm`; delta is q_heads x (packs * seq_len)
-hipError_t launch_fwd_mfma(Elem type, const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm,
-                           AttnGeom g, hipStream_t stream);
-// ds_scratch: bwd_stored_scratch_bytes(g) bytes for the one-pass backward (dS written by the dK / dV kernel, dQ formed
-// from it), or nullptr for the two-pass backward that recomputes S and dP in a dQ kernel of its own
-hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* v, const void* out, const float* lse,
-                           RowMap lm, const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g,
-                           hipStream_t stream, void* ds_scratch = nullptr);
-// 0 where the one-pass backward does not apply (head_dim other than 128, no causal mask, sparse mask, a head's blocks
-// beyond 2 GiB)
-size_t bwd_stored_scratch_bytes(const AttnGeom& g);
-
-// ---- layout adapter (layout_adapter.hip): Sentinel column layout fp32 <-> [B,H,T,d] bf16 / fp16 ----
 // Rotary embedding tables [positions][head_dim / 2] (cos == nullptr: no rotation); token t of a pack uses
 // table row offset + t.
 struct RopeTables {
@@ -79,6 +64,37 @@ struct RopeTables {
     int offset;
 };
 
+// A result tensor in Sentinel's column layout, fp32 [(head * head_dim + dim), column], for the MFMA kernels to write
+// straight from their accumulators (base == nullptr: none).  The kernels hold results transposed, one head dim of 32
+// consecutive tokens per register, which is 128 contiguous bytes of a row of that matrix: no conversion pass is
+// needed on the way out.  `base` is already advanced to the first column of pack 0; pack p starts seq_len columns on.
+// `inverse_rope`: the rotary embedding's inverse applied on the way (dQ, dK), as bhtd_to_columns does.
+struct ColumnSink {
+    float* base;
+    long long stride;  // columns per row
+    RopeTables inverse_rope;
+};
+constexpr ColumnSink kNoColumnSink = {nullptr, 0, {nullptr, nullptr, 0}};
+
+// ---- MFMA path (flash_mfma_*.hip): bf16 / fp16 [B,H,T,d] tensors, head_dim 64 or 128 ----
+bool mfma_supported(int head_dim);
+// lse rows are addressed through `lm`; delta is q_heads x (packs * seq_len).
+// out_columns: O is written there as well (the 16-bit `out` is always written: the backward reads it)
+hipError_t launch_fwd_mfma(Elem type, const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm,
+                           AttnGeom g, hipStream_t stream, ColumnSink out_columns = kNoColumnSink);
+// ds_scratch: bwd_stored_scratch_bytes(g) bytes for the one-pass backward (dS written by the dK / dV kernel, dQ formed
+// from it), or nullptr for the two-pass backward that recomputes S and dP in a dQ kernel of its own.
+// dq_columns / dk_columns / dv_columns: where given, that gradient goes there instead of to its 16-bit tensor (which may
+// then be nullptr); the one-pass backward does not take them.
+hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* v, const void* out, const float* lse,
+                           RowMap lm, const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g,
+                           hipStream_t stream, void* ds_scratch = nullptr, ColumnSink dq_columns = kNoColumnSink,
+                           ColumnSink dk_columns = kNoColumnSink, ColumnSink dv_columns = kNoColumnSink);
+// 0 where the one-pass backward does not apply (head_dim other than 128, no causal mask, sparse mask, a head's blocks
+// beyond 2 GiB)
+size_t bwd_stored_scratch_bytes(const AttnGeom& g);
+
+// ---- layout adapter (layout_adapter.hip): Sentinel column layout fp32 <-> [B,H,T,d] bf16 / fp16 ----
 hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int heads, int head_dim, int stride_columns,
                                   int seq_len, int packs, RopeTables rope, hipStream_t stream);
 hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,

@@ -34,6 +34,19 @@ constexpr int kBwdThreads = 256;
 constexpr int kSchedValu = 0x402;  // VALU and transcendental
 constexpr int kSchedMfma = 0x008;
 constexpr int kSchedDsRead = 0x100;
+
+// A wavefront's 32 x D block of a gradient goes to the caller's fp32 column matrix (rotated back where the sink carries
+// rotary tables); `head` is the tensor's head index, `token0` the block's first token inside pack `pack`.
+template <int D>
+__device__ __forceinline__ void store_block_to_sink(const f32x16 (&acc)[D / 32], float factor, const ColumnSink& sink, int head,
+                                                    int pack, int token0, int seq_len, int lane) {
+    float* head_rows = sink.base + (long long)head * D * sink.stride + (long long)pack * seq_len + token0;
+    if (sink.inverse_rope.cos)
+        store_columns_f32<D, true>(acc, factor, head_rows, (int)sink.stride, seq_len - token0, lane, sink.inverse_rope.cos,
+                                   sink.inverse_rope.sin, sink.inverse_rope.offset + token0);
+    else
+        store_columns_f32<D, false>(acc, factor, head_rows, (int)sink.stride, seq_len - token0, lane, nullptr, nullptr, 0);
+}
 constexpr int kOperandLead = 4;
 
 // ------------------------------------------------------------------------------------------------
@@ -51,7 +64,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                                                                   const float* __restrict__ lse,
                                                                   float* __restrict__ delta,
                                                                   unsigned short* __restrict__ dq, RowMap lm, AttnGeom g,
-                                                                  int q_tiles, int total_tiles, int tiles_per_xcd, int deal) {
+                                                                  int q_tiles, int total_tiles, int tiles_per_xcd, int deal,
+                                                                  ColumnSink dq_columns) {
     constexpr int KT = kDqKeyTile;
     typedef DirectTile<KT, D, kBwdThreads> Tile;
     constexpr int KSTEPS = D / 16;
@@ -292,8 +306,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 
     // dQ rows leave through the second LDS stage, which no wavefront reads or fills any more: the last trip ended with
     // a barrier, and the next tile's first loads go to stage 0 and are followed by a barrier before stage 1 is filled
-    store_rows_via_lds<E, D>(acc, g.scale, (wave < 2 ? k_lds1 : v_lds1) + (wave & 1) * (32 * D),
-                             dq + q_head + (long long)q0w * D, T - q0w, lane);
+    if (dq_columns.base)
+        store_block_to_sink<D>(acc, g.scale, dq_columns, h, b, q0w, T, lane);
+    else
+        store_rows_via_lds<E, D>(acc, g.scale, (wave < 2 ? k_lds1 : v_lds1) + (wave & 1) * (32 * D),
+                                 dq + q_head + (long long)q0w * D, T - q0w, lane);
     }  // next tile of this workgroup (the last trip ended with a barrier: the LDS stages are free)
 }
 
@@ -669,7 +686,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
-    int total_tiles, int tiles_per_xcd, int deal) {
+    int total_tiles, int tiles_per_xcd, int deal, ColumnSink dk_columns, ColumnSink dv_columns) {
     constexpr int QT = kDkvQueryTile;
     typedef RowTile<QT, D, kBwdThreads, DkvLds<D>::kPad> RTile;
     constexpr int QS = RTile::kStride;
@@ -891,9 +908,16 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
         // tile fills stage 0 and passes a barrier before it touches stage 1), one after the other through the same area
         static_assert(sizeof(DkvLds<D>) >= 4 * 32 * D * 2, "second stage too small to stage the result rows");
         unsigned short* area = reinterpret_cast<unsigned short*>(&lds[1]) + wave * (32 * D);
-        store_rows_via_lds<E, D>(dk_acc, g.scale, area, dk + kv_head + (long long)k0w * D, T - k0w, lane);
-        __builtin_amdgcn_wave_barrier();
-        store_rows_via_lds<E, D>(dv_acc, 1.0f, area, dv + kv_head + (long long)k0w * D, T - k0w, lane);
+        if (dk_columns.base) {
+            store_block_to_sink<D>(dk_acc, g.scale, dk_columns, kvh, b, k0w, T, lane);
+        } else {
+            store_rows_via_lds<E, D>(dk_acc, g.scale, area, dk + kv_head + (long long)k0w * D, T - k0w, lane);
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (dv_columns.base)
+            store_block_to_sink<D>(dv_acc, 1.0f, dv_columns, kvh, b, k0w, T, lane);
+        else
+            store_rows_via_lds<E, D>(dv_acc, 1.0f, area, dv + kv_head + (long long)k0w * D, T - k0w, lane);
     }
     }  // next key tile of this workgroup (every stage trip ended with a barrier: the LDS stages are free)
 }
@@ -903,7 +927,8 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
-    int total_tiles, int tiles_per_xcd, int deal, unsigned short* __restrict__ ds_out) {
+    int total_tiles, int tiles_per_xcd, int deal, unsigned short* __restrict__ ds_out, ColumnSink dk_columns,
+    ColumnSink dv_columns) {
     static_assert(!(STORE_DS && WINDOW), "the stored score gradients cover the full causal / full rectangle only");
     constexpr int QT = kDkvQueryTile;
     // the query / dO tiles of a stage are staged by the score wavefronts alone (threads 0..255): they have about a
@@ -1258,9 +1283,12 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         if constexpr (STORE_DS) {
             if (n_iter >= 2) flush_ds(n_iter & 1);  // dS of the last stage but one still sits in that buffer
         }
-        store_rows_via_lds<E, D, true, 16>(
-            acc, 1.0f, reinterpret_cast<unsigned short*>(dkv_smem + kPBase + (n_iter & 1) * kPBufBytes) + kblock * (16 * D),
-            dv + kv_head + (long long)k0w * D, T - k0w, lane);
+        if (dv_columns.base)
+            store_block_to_sink<D>(acc, 1.0f, dv_columns, kvh, b, k0w, T, lane);
+        else
+            store_rows_via_lds<E, D, true, 16>(
+                acc, 1.0f, reinterpret_cast<unsigned short*>(dkv_smem + kPBase + (n_iter & 1) * kPBufBytes) + kblock * (16 * D),
+                dv + kv_head + (long long)k0w * D, T - k0w, lane);
         __syncthreads();
         if constexpr (STORE_DS) flush_ds((n_iter - 1) & 1);  // the last stage's dS, complete with this barrier
     } else {
@@ -1273,7 +1301,10 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         // next key tile fills stage 0 and passes a barrier before it touches the others
         static_assert(2 * sizeof(DkvSplitStage<D>) >= 4 * 32 * D * 2, "stages 1 and 2 too small to stage the dK rows");
         unsigned short* area = reinterpret_cast<unsigned short*>(dkv_smem + sizeof(DkvSplitStage<D>)) + kblock * (32 * D);
-        store_rows_via_lds<E, D>(acc, g.scale, area, dk + kv_head + (long long)k0w * D, T - k0w, lane);
+        if (dk_columns.base)
+            store_block_to_sink<D>(acc, g.scale, dk_columns, kvh, b, k0w, T, lane);
+        else
+            store_rows_via_lds<E, D>(acc, g.scale, area, dk + kv_head + (long long)k0w * D, T - k0w, lane);
     }
     }  // next key tile of this workgroup (both roles have passed the last barrier of the tile: the LDS is free)
 }
@@ -1307,7 +1338,7 @@ hipError_t run_bwd_stored(const unsigned short* qp, const unsigned short* kp, co
             const int grid = kXcds * (tiles_per_xcd < resident ? tiles_per_xcd : resident);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp, dvp, lm, g,
-                               k_tiles, total, tiles_per_xcd, 0, ds);
+                               k_tiles, total, tiles_per_xcd, 0, ds, kNoColumnSink, kNoColumnSink);
             return hipGetLastError();
         };
         const hipError_t err = launch(dkdv_split_kernel<E, D, true, false, true>);
@@ -1328,7 +1359,7 @@ hipError_t run_bwd_stored(const unsigned short* qp, const unsigned short* kp, co
 template <typename E, int D>
 hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse, RowMap lm,
                    const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g, void* ds_scratch,
-                   hipStream_t stream) {
+                   hipStream_t stream, ColumnSink dq_columns, ColumnSink dk_columns, ColumnSink dv_columns) {
     auto qp = static_cast<const unsigned short*>(q);
     auto kp = static_cast<const unsigned short*>(k);
     auto vp = static_cast<const unsigned short*>(v);
@@ -1339,7 +1370,7 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
     auto dvp = static_cast<unsigned short*>(dv);
     const int T = g.seq_len;
     if constexpr (D == 128) {
-        if (ds_scratch)
+        if (ds_scratch && !dq_columns.base && !dk_columns.base && !dv_columns.base)
             return run_bwd_stored<E, D>(qp, kp, vp, op, lse, lm, gp, dqp, dkp, dvp, delta, g,
                                         static_cast<unsigned short*>(ds_scratch), stream);
     }
@@ -1359,7 +1390,7 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
                                                : plan_persistent_grid(total, q_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dq_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp, lse, delta, dqp,
-                               lm, g, q_tiles, total, tiles_per_xcd, plan.deal);
+                               lm, g, q_tiles, total, tiles_per_xcd, plan.deal, dq_columns);
         };
         if (g.window > 0)
             launch(dq_mfma_kernel<E, D, true, true>);
@@ -1385,7 +1416,7 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
                                                : plan_persistent_grid(total, k_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kBwdThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp,
-                               dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal);
+                               dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal, dk_columns, dv_columns);
         };
         if (g.window > 0)
             launch(dkdv_mfma_kernel<E, D, true, true>);
@@ -1408,7 +1439,8 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
                                                : plan_persistent_grid(total, k_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp,
-                               dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal, static_cast<unsigned short*>(nullptr));
+                               dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal, static_cast<unsigned short*>(nullptr),
+                               dk_columns, dv_columns);
             return hipGetLastError();
         };
         if (g.window > 0)
@@ -1433,14 +1465,19 @@ size_t bwd_stored_scratch_bytes(const AttnGeom& g) {
 
 hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* v, const void* out, const float* lse,
                            RowMap lm, const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g,
-                           hipStream_t stream, void* ds_scratch) {
+                           hipStream_t stream, void* ds_scratch, ColumnSink dq_columns, ColumnSink dk_columns,
+                           ColumnSink dv_columns) {
     if (ds_scratch && bwd_stored_scratch_bytes(g) == 0) ds_scratch = nullptr;
     if (type == Elem::BF16) {
-        if (g.head_dim == 64) return run_bwd<Bf16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream);
-        if (g.head_dim == 128) return run_bwd<Bf16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream);
+        if (g.head_dim == 64) return run_bwd<Bf16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream, dq_columns, dk_columns,
+                                                              dv_columns);
+        if (g.head_dim == 128) return run_bwd<Bf16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream, dq_columns, dk_columns,
+                                                              dv_columns);
     } else if (type == Elem::F16) {
-        if (g.head_dim == 64) return run_bwd<Fp16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream);
-        if (g.head_dim == 128) return run_bwd<Fp16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream);
+        if (g.head_dim == 64) return run_bwd<Fp16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream, dq_columns, dk_columns,
+                                                              dv_columns);
+        if (g.head_dim == 128) return run_bwd<Fp16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream, dq_columns, dk_columns,
+                                                              dv_columns);
     }
     return hipErrorInvalidValue;
 }

@@ -41,7 +41,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
                                                                    const unsigned short* __restrict__ v,
                                                                    unsigned short* __restrict__ out,
                                                                    float* __restrict__ lse, RowMap lm, AttnGeom g,
-                                                                   int q_tiles, int total_tiles, int tiles_per_xcd, int deal) {
+                                                                   int q_tiles, int total_tiles, int tiles_per_xcd, int deal,
+                                                                   ColumnSink out_columns) {
     constexpr int KT = kFwdKeyTile;
     typedef DirectTile<KT, D, kFwdThreads> Tile;
     constexpr int KSTEPS = D / 16;  // k-steps of the S^T product
@@ -289,6 +290,10 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
     // barrier, and the next tile's first loads go to stage 0 and are followed by a barrier before stage 1 is filled
     store_rows_via_lds<E, D, false>(acc, inv, (wave < 2 ? k_lds1 : v_lds1) + (wave & 1) * (32 * D),
                              out + ((long long)b * g.q_heads + h) * T * D + (long long)q0w * D, T - q0w, lane);
+    // the caller's fp32 column matrix, if it keeps O that way: straight from the accumulators, unrounded
+    if (out_columns.base)
+        store_columns_f32<D, false>(acc, inv, out_columns.base + (long long)h * D * out_columns.stride + (long long)b * T + q0w,
+                                    (int)out_columns.stride, T - q0w, lane, nullptr, nullptr, 0);
     if (qrow < T && gh == 0)
         lse[b * lm.pack_stride + h * lm.head_stride + qrow] = m_run * g.scale + (l_tot > 0.0f ? __logf(l_tot) : 0.0f);
     }  // next tile of this workgroup (the last trip ended with a barrier: the LDS stages are free)
@@ -296,7 +301,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned
 
 template <typename E, int D>
 hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm, AttnGeom g,
-                   hipStream_t stream) {
+                   hipStream_t stream, ColumnSink out_columns) {
     const int q_tiles = (g.seq_len + kFwdQueryTile - 1) / kFwdQueryTile;
     const int total = g.packs * g.q_heads * q_tiles;
     const int tiles_per_xcd = (total + kXcds - 1) / kXcds;
@@ -313,7 +318,7 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
                                            : plan_persistent_grid(total, q_tiles, resident, g.causal != 0, streamed);
         KernelTimer timer("fwd_mfma", stream);
         hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm, g, q_tiles,
-                           total, tiles_per_xcd, plan.deal);
+                           total, tiles_per_xcd, plan.deal, out_columns);
     };
     if (g.window > 0)
         launch(fwd_mfma_kernel<E, D, true, true>);
@@ -329,13 +334,13 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
 bool mfma_supported(int head_dim) { return head_dim == 64 || head_dim == 128; }
 
 hipError_t launch_fwd_mfma(Elem type, const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm,
-                           AttnGeom g, hipStream_t stream) {
+                           AttnGeom g, hipStream_t stream, ColumnSink out_columns) {
     if (type == Elem::BF16) {
-        if (g.head_dim == 64) return run_fwd<Bf16, 64>(q, k, v, out, lse, lm, g, stream);
-        if (g.head_dim == 128) return run_fwd<Bf16, 128>(q, k, v, out, lse, lm, g, stream);
+        if (g.head_dim == 64) return run_fwd<Bf16, 64>(q, k, v, out, lse, lm, g, stream, out_columns);
+        if (g.head_dim == 128) return run_fwd<Bf16, 128>(q, k, v, out, lse, lm, g, stream, out_columns);
     } else if (type == Elem::F16) {
-        if (g.head_dim == 64) return run_fwd<Fp16, 64>(q, k, v, out, lse, lm, g, stream);
-        if (g.head_dim == 128) return run_fwd<Fp16, 128>(q, k, v, out, lse, lm, g, stream);
+        if (g.head_dim == 64) return run_fwd<Fp16, 64>(q, k, v, out, lse, lm, g, stream, out_columns);
+        if (g.head_dim == 128) return run_fwd<Fp16, 128>(q, k, v, out, lse, lm, g, stream, out_columns);
     }
     return hipErrorInvalidValue;
 }

@@ -305,6 +305,59 @@ __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], 
 // round-robin to them, so workgroup id % kXcds names the die a workgroup runs on.
 constexpr int kXcds = 8;
 
+// Writes a wavefront's 32 x D block of fp32 results into a column-layout matrix [(head * D + dim), column] (see
+// ColumnSink).  The block is held as transposed accumulators: lane (n, gh) owns token n, head dims
+// cb*32 + a*8 + gh*4 + [0, 4) in acc[cb][a*4 + ...]; one store instruction writes one head dim of 32 consecutive tokens
+// (128 contiguous bytes) for each lane half.  `head_rows` points at (dim 0 of the head, the block's first token).
+// Buffer stores: the per-lane part of the address (token, lane half) is one register for all 16 * D / 32 stores, the head
+// dim's row is a scalar offset; D * stride * 4 must stay below 2^31 (the host checks).
+// ROTATE: each (even, odd) pair of head dims is rotated back by the angle of its token's position (table row
+// `position0 + n`), in fp32 without fused multiply-adds, exactly as the conversion pass bhtd_to_columns does.
+template <int D, bool ROTATE>
+__device__ __forceinline__ void store_columns_f32(const f32x16 (&acc)[D / 32], float factor, float* head_rows, int stride,
+                                                  int valid_rows, int lane, const float* cos_table, const float* sin_table,
+                                                  int position0) {
+#pragma clang fp contract(off)
+    const int n = lane % 32;
+    const int gh = lane / 32;
+    if (n >= valid_rows) return;
+    const __amdgpu_buffer_rsrc_t rows = __builtin_amdgcn_make_buffer_rsrc(head_rows, 0, 0x7fffffff, 0x00020000);
+    const int lane_bytes = (gh * 4 * stride + n) * 4;
+    __amdgpu_buffer_rsrc_t cos_rows = rows, sin_rows = rows;
+    int table_bytes = 0;
+    if (ROTATE) {
+        cos_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(cos_table) + (long long)position0 * (D / 2), 0, 0x7fffffff,
+                                                     0x00020000);
+        sin_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sin_table) + (long long)position0 * (D / 2), 0, 0x7fffffff,
+                                                     0x00020000);
+        table_bytes = (n * (D / 2) + gh * 2) * 4;
+    }
+#pragma unroll
+    for (int cb = 0; cb < D / 32; ++cb)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int dim = cb * 32 + a * 8;  // + gh * 4 through the lane's offset
+            float x[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) x[j] = acc[cb][a * 4 + j] * factor;
+            if (ROTATE) {
+                // (two 32-bit loads per table: the 64-bit buffer load builtin of this toolchain fetches one word only)
+                const float c0 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cos_rows, table_bytes, (dim / 2) * 4, 0));
+                const float c1 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cos_rows, table_bytes, (dim / 2) * 4 + 4, 0));
+                const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sin_rows, table_bytes, (dim / 2) * 4, 0));
+                const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sin_rows, table_bytes, (dim / 2) * 4 + 4, 0));
+                const float e0 = x[0], o0 = x[1], e1 = x[2], o1 = x[3];
+                x[0] = e0 * c0 + o0 * s0;
+                x[1] = -e0 * s0 + o0 * c0;
+                x[2] = e1 * c1 + o1 * s1;
+                x[3] = -e1 * s1 + o1 * c1;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[j]), rows, lane_bytes, (dim + j) * stride * 4, 0);
+        }
+}
+
 // Which tile of its XCD a workgroup of a persistent grid takes in `round`.  The XCD's tiles are numbered head-major,
 // the longest tile of a head first (the last query tile, or the first key tile, under the causal mask);
 // `slot` = workgroup id / kXcds of `slots`.
