@@ -36,7 +36,7 @@ constexpr int kOperandLead = 4;
 constexpr int kFwdKeyTile = 64;
 
 template <typename E, int D, bool CAUSAL, bool WINDOW>
-__global__ __launch_bounds__(kFwdThreads, 2) void fwd_mfma_kernel(const unsigned short* __restrict__ q,
+__global__ __launch_bounds__(kFwdThreads, D <= 64 ? 3 : 2) void fwd_mfma_kernel(const unsigned short* __restrict__ q,
                                                                    const unsigned short* __restrict__ k,
                                                                    const unsigned short* __restrict__ v,
                                                                    unsigned short* __restrict__ out,

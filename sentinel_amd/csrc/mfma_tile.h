@@ -318,6 +318,7 @@ __device__ __forceinline__ void store_columns_f32(const f32x16 (&acc)[D / 32], f
                                                   int valid_rows, int lane, const float* cos_table, const float* sin_table,
                                                   int position0) {
 #pragma clang fp contract(off)
+    asm volatile("" : "+v"(lane));  // keeps the per-lane address arithmetic here instead of hoisted over the caller's loops
     const int n = lane % 32;
     const int gh = lane / 32;
     if (n >= valid_rows) return;
