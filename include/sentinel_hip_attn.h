@@ -63,6 +63,9 @@ enum {
  *        element(head, dim, column) = base[(head * head_dim + dim) * stride_columns + column]
  *        pack p occupies columns [column_start + p * seq_len, column_start + (p + 1) * seq_len);
  *        lse is q_heads x stride_columns. Columns outside the pack window are never written.
+ *        With 16-bit arithmetic the operands are converted into the workspace by passes of their own; the results
+ *        (out, dq, dk, dv) are written by the attention kernels themselves, as the fp32 values of their accumulators
+ *        (rounded to the arithmetic type they equal the BHTD layout's results).
  *  SENTINEL_HIP_LAYOUT_BHTD     contiguous [pack_count, heads, seq_len, head_dim]; lse is
  *        [pack_count, q_heads, seq_len]; stride_columns and column_start are ignored.
  * delta workspace (both layouts): q_heads x (pack_count * seq_len) floats, the shape the CUDA caller
@@ -74,7 +77,7 @@ enum { SENTINEL_HIP_LAYOUT_COLUMNS = 0, SENTINEL_HIP_LAYOUT_BHTD = 1 };
  * Workspace flags, OR-ed into the `layout` argument. They matter where a workspace is used at all (COLUMNS layout with
  * MFMA arithmetic) and are ignored elsewhere. The CUDA layer keeps flashLogSumExp from its forward call for its
  * backward call (CudaCausalSelfAttention.cu:237-249, :421-438); a caller that keeps the workspace the same way saves
- * the backward four of its conversion passes:
+ * the backward four of its five conversion passes:
  *  SENTINEL_HIP_WORKSPACE_KEEP   forward: `workspace` is sized for the BACKWARD call
  *        (sentinel_hip_flash_workspace_bytes(..., backward = 1)) and the 16-bit copies of q, k, v (rotated, if the call
  *        rotates) and out are left in it where the backward call looks for them.
