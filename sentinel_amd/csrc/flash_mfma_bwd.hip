@@ -55,7 +55,9 @@ constexpr int kOperandLead = 4;
 constexpr int kDqQueryTile = 128;
 constexpr int kDqKeyTile = 64;
 
-template <typename E, int D, bool CAUSAL, bool WINDOW>
+// COLUMNS: dQ goes to the caller's fp32 column matrix (dq_columns) instead of the 16-bit tensor; a compile-time switch,
+// because with the choice made at run time the 16-bit version lost 1.5 - 2 %.
+template <typename E, int D, bool CAUSAL, bool WINDOW, bool COLUMNS = false>
 __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned short* __restrict__ q,
                                                                   const unsigned short* __restrict__ k,
                                                                   const unsigned short* __restrict__ v,
@@ -306,7 +308,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 
     // dQ rows leave through the second LDS stage, which no wavefront reads or fills any more: the last trip ended with
     // a barrier, and the next tile's first loads go to stage 0 and are followed by a barrier before stage 1 is filled
-    if (dq_columns.base)
+    if constexpr (COLUMNS)
         store_block_to_sink<D>(acc, g.scale, dq_columns, h, b, q0w, T, lane);
     else
         store_rows_via_lds<E, D>(acc, g.scale, (wave < 2 ? k_lds1 : v_lds1) + (wave & 1) * (32 * D),
@@ -923,7 +925,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     }  // next key tile of this workgroup (every stage trip ended with a barrier: the LDS stages are free)
 }
 
-template <typename E, int D, bool CAUSAL, bool WINDOW, bool STORE_DS = false>
+// COLUMNS: as in dkdv_mfma_kernel
+template <typename E, int D, bool CAUSAL, bool WINDOW, bool STORE_DS = false, bool COLUMNS = false>
 __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
@@ -1284,7 +1287,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         if constexpr (STORE_DS) {
             if (n_iter >= 2) flush_ds(n_iter & 1);  // dS of the last stage but one still sits in that buffer
         }
-        if (dv_columns.base)
+        if constexpr (COLUMNS)
             store_block_to_sink<D>(acc, 1.0f, dv_columns, kvh, b, k0w, T, lane);
         else
             store_rows_via_lds<E, D, true, 16>(
@@ -1302,7 +1305,7 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         // next key tile fills stage 0 and passes a barrier before it touches the others
         static_assert(2 * sizeof(DkvSplitStage<D>) >= 4 * 32 * D * 2, "stages 1 and 2 too small to stage the dK rows");
         unsigned short* area = reinterpret_cast<unsigned short*>(dkv_smem + sizeof(DkvSplitStage<D>)) + kblock * (32 * D);
-        if (dk_columns.base)
+        if constexpr (COLUMNS)
             store_block_to_sink<D>(acc, g.scale, dk_columns, kvh, b, k0w, T, lane);
         else
             store_rows_via_lds<E, D>(acc, g.scale, area, dk + kv_head + (long long)k0w * D, T - k0w, lane);
@@ -1393,12 +1396,13 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
             hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kBwdThreads), 0, stream, qp, kp, vp, op, gp, lse, delta, dqp,
                                lm, g, q_tiles, total, tiles_per_xcd, plan.deal, dq_columns);
         };
+        const bool columns = dq_columns.base != nullptr;
         if (g.window > 0)
-            launch(dq_mfma_kernel<E, D, true, true>);
+            columns ? launch(dq_mfma_kernel<E, D, true, true, true>) : launch(dq_mfma_kernel<E, D, true, true>);
         else if (g.causal)
-            launch(dq_mfma_kernel<E, D, true, false>);
+            columns ? launch(dq_mfma_kernel<E, D, true, false, true>) : launch(dq_mfma_kernel<E, D, true, false>);
         else
-            launch(dq_mfma_kernel<E, D, false, false>);
+            columns ? launch(dq_mfma_kernel<E, D, false, false, true>) : launch(dq_mfma_kernel<E, D, false, false>);
         err = hipGetLastError();
         if (err != hipSuccess) return err;
     }
@@ -1447,12 +1451,14 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
                                dk_columns, dv_columns);
             return hipGetLastError();
         };
+        const bool columns = dk_columns.base && dv_columns.base;
+        if (columns != (dk_columns.base || dv_columns.base)) return hipErrorInvalidValue;
         if (g.window > 0)
-            err = launch(dkdv_split_kernel<E, D, true, true>);
+            err = columns ? launch(dkdv_split_kernel<E, D, true, true, false, true>) : launch(dkdv_split_kernel<E, D, true, true>);
         else if (g.causal)
-            err = launch(dkdv_split_kernel<E, D, true, false>);
+            err = columns ? launch(dkdv_split_kernel<E, D, true, false, false, true>) : launch(dkdv_split_kernel<E, D, true, false>);
         else
-            err = launch(dkdv_split_kernel<E, D, false, false>);
+            err = columns ? launch(dkdv_split_kernel<E, D, false, false, false, true>) : launch(dkdv_split_kernel<E, D, false, false>);
     }
     return err;
 }
