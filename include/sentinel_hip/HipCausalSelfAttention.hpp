@@ -193,6 +193,12 @@ public:
     HipMatrix query, key, value, attended, output;
     HipMatrix inputCache, attendedGradient, queryGradient, keyGradient, valueGradient;
     HipMatrix flashLogSumExp, flashDelta;
+    /// the forward call's 16-bit operands, kept for the backward call like flashLogSumExp (MFMA arithmetic only; costs
+    /// 4 bytes per element of query / key / value in device memory per layer; set keepFlashOperands = false to convert
+    /// them again in the backward call instead)
+    HipFlashAttention::KeptOperands flashOperands;
+    bool keepFlashOperands = true;
+    HipFlashAttention::KeptOperands* keptOperands() { return keepFlashOperands ? &flashOperands : nullptr; }
     /// dense path: probabilities of every (head, pack), row (head * packs + pack) holds one keys x queries matrix; kept
     /// for the backward like the CUDA class's cachedHeadProbabilities
     HipMatrix probabilities;
@@ -297,6 +303,7 @@ public:
     void releaseFlashAttentionScratch() {
         flashLogSumExp = HipMatrix();
         flashDelta = HipMatrix();
+        flashOperands.release();
     }
     /// free the activations after a forward, weights kept (CudaCausalSelfAttention::releaseActivationScratch, :88-108)
     void releaseActivationScratch() {
@@ -351,11 +358,11 @@ public:
             if (sparse)
                 HipFlashAttention::forwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, &cosTable, &sinTable, 0,
                                                           windowSize, globalTokenCount, headCount, headDimension, scale, 0,
-                                                          segmentLength, activePackCount, kvHeadCount);
+                                                          segmentLength, activePackCount, kvHeadCount, keptOperands());
             else
                 HipFlashAttention::forwardMultiHeadRope(query, key, value, attended, flashLogSumExp, cosTable, sinTable, 0,
                                                         headCount, headDimension, scale, true, 0, segmentLength,
-                                                        activePackCount, kvHeadCount);
+                                                        activePackCount, kvHeadCount, keptOperands());
         } else {
             releaseDenseAttentionScratch();
             HipOps::rotaryRotateInPlace(query, headCount, headDimension, pairCount, cosTable, sinTable, 0, segmentLength);
@@ -363,10 +370,10 @@ public:
             if (sparse)
                 HipFlashAttention::forwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, nullptr, nullptr, 0,
                                                           windowSize, globalTokenCount, headCount, headDimension, scale, 0,
-                                                          segmentLength, activePackCount, kvHeadCount);
+                                                          segmentLength, activePackCount, kvHeadCount, keptOperands());
             else
                 HipFlashAttention::forwardMultiHead(query, key, value, attended, flashLogSumExp, headCount, headDimension, scale,
-                                                    true, 0, segmentLength, activePackCount, kvHeadCount);
+                                                    true, 0, segmentLength, activePackCount, kvHeadCount, keptOperands());
         }
         HipGemm::multiplyInto(outputWeight, attended, out);
     }
@@ -408,23 +415,23 @@ public:
                 HipFlashAttention::backwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, attendedGradient,
                                                            queryGradient, keyGradient, valueGradient, flashDelta, &cosTable,
                                                            &sinTable, 0, windowSize, globalTokenCount, headCount, headDimension,
-                                                           scale, 0, activeSegmentLength, activePackCount, kvHeadCount);
+                                                           scale, 0, activeSegmentLength, activePackCount, kvHeadCount, keptOperands());
             else
                 HipFlashAttention::backwardMultiHeadRope(query, key, value, attended, flashLogSumExp, attendedGradient,
                                                          queryGradient, keyGradient, valueGradient, flashDelta, cosTable,
                                                          sinTable, 0, headCount, headDimension, scale, true, 0,
-                                                         activeSegmentLength, activePackCount, kvHeadCount);
+                                                         activeSegmentLength, activePackCount, kvHeadCount, keptOperands());
         } else {
             if (sparse)
                 HipFlashAttention::backwardMultiHeadSparse(query, key, value, attended, flashLogSumExp, attendedGradient,
                                                            queryGradient, keyGradient, valueGradient, flashDelta, nullptr,
                                                            nullptr, 0, windowSize, globalTokenCount, headCount, headDimension,
-                                                           scale, 0, activeSegmentLength, activePackCount, kvHeadCount);
+                                                           scale, 0, activeSegmentLength, activePackCount, kvHeadCount, keptOperands());
             else
                 HipFlashAttention::backwardMultiHead(query, key, value, attended, flashLogSumExp, attendedGradient,
                                                      queryGradient, keyGradient, valueGradient, flashDelta, headCount,
                                                      headDimension, scale, true, 0, activeSegmentLength, activePackCount,
-                                                     kvHeadCount);
+                                                     kvHeadCount, keptOperands());
             HipOps::rotaryRotateInverseInPlace(queryGradient, headCount, headDimension, pairCount, cosTable, sinTable, 0,
                                                activeSegmentLength);
             HipOps::rotaryRotateInverseInPlace(keyGradient, kvHeadCount, headDimension, pairCount, cosTable, sinTable, 0,

@@ -137,6 +137,23 @@ public:
         return stream;
     }
 
+    /// The 16-bit copies of query, key, value and out that a forward call with MFMA arithmetic makes anyway, kept for the
+    /// backward call of the same tensors (SENTINEL_HIP_WORKSPACE_KEEP / _REUSE), the way CudaCausalSelfAttention keeps
+    /// flashLogSumExp between its two calls (Cuda/CudaCausalSelfAttention.cu:237-249, :421-438): the backward call then
+    /// converts outGradient only. One per layer; pass it to the forward and to the backward call. A backward call whose
+    /// shape, window, arithmetic or rotation differs from the forward call that filled it converts everything again.
+    struct KeptOperands {
+        HipDeviceBuffer workspace;
+        bool filled = false;
+        const void* query = nullptr;
+        const void* tables = nullptr;
+        int geometry[11] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        void release() {
+            workspace.free();
+            filled = false;
+        }
+    };
+
     static void forward(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, HipMatrix& out,
                         HipMatrix& logSumExp, float scale, bool causal = true) {
         forwardMultiHead(query, key, value, out, logSumExp, 1, static_cast<int>(query.rows), scale, causal, 0,
@@ -145,17 +162,20 @@ public:
 
     static void forwardMultiHead(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, HipMatrix& out,
                                  HipMatrix& logSumExp, int headCount, int headDimension, float scale, bool causal = true,
-                                 int columnStart = 0, int columnCount = 0, int packCount = 1, int kvHeadCount = 0) {
+                                 int columnStart = 0, int columnCount = 0, int packCount = 1, int kvHeadCount = 0,
+                                 KeptOperands* kept = nullptr) {
         const char* op = "HipFlashAttention::forwardMultiHead";
         const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
         if (!sentinel_hip_device_available()) throw std::runtime_error(std::string(op) + " no HIP device");
         out.ensureSize(query.rows, query.cols);
         logSumExp.ensureSize(static_cast<size_t>(headCount), query.cols);
         void* ws = nullptr;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws);
+        int layoutFlags = 0;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws,
+                                            kept, nullptr, 0, 0, 0, layoutFlags);
         check(sentinel_hip_flash_fwd(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                      out.buffer.deviceData, logSumExp.buffer.deviceData, SENTINEL_HIP_F32, computeType(),
-                                     SENTINEL_HIP_LAYOUT_COLUMNS, headCount, kvHeads, headDimension,
+                                     SENTINEL_HIP_LAYOUT_COLUMNS | layoutFlags, headCount, kvHeads, headDimension,
                                      static_cast<int>(query.cols), columnStart, columnCount, packCount, scale, causal ? 1 : 0,
                                      ws, wsBytes, activeStream()));
     }
@@ -173,7 +193,7 @@ public:
                                   const HipMatrix& logSumExp, const HipMatrix& outGradient, HipMatrix& queryGradient,
                                   HipMatrix& keyGradient, HipMatrix& valueGradient, HipMatrix& deltaWorkspace, int headCount,
                                   int headDimension, float scale, bool causal = true, int columnStart = 0,
-                                  int columnCount = 0, int packCount = 1, int kvHeadCount = 0) {
+                                  int columnCount = 0, int packCount = 1, int kvHeadCount = 0, KeptOperands* kept = nullptr) {
         const char* op = "HipFlashAttention::backwardMultiHead";
         const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
         if (out.rows != query.rows || out.cols != query.cols) throw std::invalid_argument(std::string(op) + " out shape mismatch");
@@ -191,12 +211,14 @@ public:
         valueGradient.ensureSize(value.rows, value.cols);
         deltaWorkspace.ensureSize(static_cast<size_t>(headCount), static_cast<size_t>(packCount) * static_cast<size_t>(resolvedCount));
         void* ws = nullptr;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws);
+        int layoutFlags = 0;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws,
+                                            kept, nullptr, 0, 0, 0, layoutFlags);
         check(sentinel_hip_flash_bwd(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                      out.buffer.deviceData, logSumExp.buffer.deviceData, outGradient.buffer.deviceData,
                                      queryGradient.buffer.deviceData, keyGradient.buffer.deviceData,
                                      valueGradient.buffer.deviceData, deltaWorkspace.buffer.deviceData, SENTINEL_HIP_F32,
-                                     computeType(), SENTINEL_HIP_LAYOUT_COLUMNS, headCount, kvHeads, headDimension,
+                                     computeType(), SENTINEL_HIP_LAYOUT_COLUMNS | layoutFlags, headCount, kvHeads, headDimension,
                                      static_cast<int>(query.cols), columnStart, columnCount, packCount, scale, causal ? 1 : 0,
                                      ws, wsBytes, activeStream()));
     }
@@ -206,7 +228,8 @@ public:
     static void forwardMultiHeadRope(const HipMatrix& query, const HipMatrix& key, const HipMatrix& value, HipMatrix& out,
                                      HipMatrix& logSumExp, const HipMatrix& cosTable, const HipMatrix& sinTable,
                                      int positionOffset, int headCount, int headDimension, float scale, bool causal = true,
-                                     int columnStart = 0, int columnCount = 0, int packCount = 1, int kvHeadCount = 0) {
+                                     int columnStart = 0, int columnCount = 0, int packCount = 1, int kvHeadCount = 0,
+                                 KeptOperands* kept = nullptr) {
         const char* op = "HipFlashAttention::forwardMultiHeadRope";
         const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
         if (cosTable.empty() || sinTable.empty()) throw std::invalid_argument(std::string(op) + " empty tables");
@@ -214,11 +237,13 @@ public:
         out.ensureSize(query.rows, query.cols);
         logSumExp.ensureSize(static_cast<size_t>(headCount), query.cols);
         void* ws = nullptr;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws);
+        int layoutFlags = 0;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws,
+                                            kept, cosTable.buffer.deviceData, 0, 0, positionOffset, layoutFlags);
         check(sentinel_hip_flash_fwd_rope(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                           out.buffer.deviceData, logSumExp.buffer.deviceData, cosTable.buffer.deviceData,
                                           sinTable.buffer.deviceData, static_cast<int>(cosTable.rows), positionOffset,
-                                          SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS, headCount, kvHeads,
+                                          SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS | layoutFlags, headCount, kvHeads,
                                           headDimension, static_cast<int>(query.cols), columnStart, columnCount, packCount,
                                           scale, causal ? 1 : 0, ws, wsBytes, activeStream()));
     }
@@ -229,7 +254,7 @@ public:
                                       HipMatrix& keyGradient, HipMatrix& valueGradient, HipMatrix& deltaWorkspace,
                                       const HipMatrix& cosTable, const HipMatrix& sinTable, int positionOffset, int headCount,
                                       int headDimension, float scale, bool causal = true, int columnStart = 0,
-                                      int columnCount = 0, int packCount = 1, int kvHeadCount = 0) {
+                                      int columnCount = 0, int packCount = 1, int kvHeadCount = 0, KeptOperands* kept = nullptr) {
         const char* op = "HipFlashAttention::backwardMultiHeadRope";
         const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
         if (out.rows != query.rows || out.cols != query.cols) throw std::invalid_argument(std::string(op) + " out shape mismatch");
@@ -248,14 +273,16 @@ public:
         valueGradient.ensureSize(value.rows, value.cols);
         deltaWorkspace.ensureSize(static_cast<size_t>(headCount), static_cast<size_t>(packCount) * static_cast<size_t>(resolvedCount));
         void* ws = nullptr;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws);
+        int layoutFlags = 0;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws,
+                                            kept, cosTable.buffer.deviceData, 0, 0, positionOffset, layoutFlags);
         check(sentinel_hip_flash_bwd_rope(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                           out.buffer.deviceData, logSumExp.buffer.deviceData, outGradient.buffer.deviceData,
                                           queryGradient.buffer.deviceData, keyGradient.buffer.deviceData,
                                           valueGradient.buffer.deviceData, deltaWorkspace.buffer.deviceData,
                                           cosTable.buffer.deviceData, sinTable.buffer.deviceData,
                                           static_cast<int>(cosTable.rows), positionOffset, SENTINEL_HIP_F32, computeType(),
-                                          SENTINEL_HIP_LAYOUT_COLUMNS, headCount, kvHeads, headDimension,
+                                          SENTINEL_HIP_LAYOUT_COLUMNS | layoutFlags, headCount, kvHeads, headDimension,
                                           static_cast<int>(query.cols), columnStart, columnCount, packCount, scale,
                                           causal ? 1 : 0, ws, wsBytes, activeStream()));
     }
@@ -267,7 +294,7 @@ public:
                                        HipMatrix& logSumExp, const HipMatrix* cosTable, const HipMatrix* sinTable,
                                        int positionOffset, int windowSize, int globalTokenCount, int headCount,
                                        int headDimension, float scale, int columnStart = 0, int columnCount = 0,
-                                       int packCount = 1, int kvHeadCount = 0) {
+                                       int packCount = 1, int kvHeadCount = 0, KeptOperands* kept = nullptr) {
         const char* op = "HipFlashAttention::forwardMultiHeadSparse";
         const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
         if ((cosTable == nullptr) != (sinTable == nullptr)) throw std::invalid_argument(std::string(op) + " empty tables");
@@ -276,13 +303,15 @@ public:
         out.ensureSize(query.rows, query.cols);
         logSumExp.ensureSize(static_cast<size_t>(headCount), query.cols);
         void* ws = nullptr;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws);
+        int layoutFlags = 0;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws,
+                                            kept, cosTable ? cosTable->buffer.deviceData : nullptr, windowSize, globalTokenCount, positionOffset, layoutFlags);
         check(sentinel_hip_flash_fwd_sparse(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                             out.buffer.deviceData, logSumExp.buffer.deviceData,
                                             cosTable ? cosTable->buffer.deviceData : nullptr,
                                             sinTable ? sinTable->buffer.deviceData : nullptr,
                                             cosTable ? static_cast<int>(cosTable->rows) : 0, positionOffset, windowSize,
-                                            globalTokenCount, SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS,
+                                            globalTokenCount, SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS | layoutFlags,
                                             headCount, kvHeads, headDimension, static_cast<int>(query.cols), columnStart,
                                             columnCount, packCount, scale, 1, ws, wsBytes, activeStream()));
     }
@@ -294,7 +323,7 @@ public:
                                         HipMatrix& deltaWorkspace, const HipMatrix* cosTable, const HipMatrix* sinTable,
                                         int positionOffset, int windowSize, int globalTokenCount, int headCount,
                                         int headDimension, float scale, int columnStart = 0, int columnCount = 0,
-                                        int packCount = 1, int kvHeadCount = 0) {
+                                        int packCount = 1, int kvHeadCount = 0, KeptOperands* kept = nullptr) {
         const char* op = "HipFlashAttention::backwardMultiHeadSparse";
         const int kvHeads = validateMultiHeadShape(query, key, value, headCount, headDimension, kvHeadCount, op);
         if (out.rows != query.rows || out.cols != query.cols) throw std::invalid_argument(std::string(op) + " out shape mismatch");
@@ -314,7 +343,9 @@ public:
         valueGradient.ensureSize(value.rows, value.cols);
         deltaWorkspace.ensureSize(static_cast<size_t>(headCount), static_cast<size_t>(packCount) * static_cast<size_t>(resolvedCount));
         void* ws = nullptr;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws);
+        int layoutFlags = 0;
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws,
+                                            kept, cosTable ? cosTable->buffer.deviceData : nullptr, windowSize, globalTokenCount, positionOffset, layoutFlags);
         check(sentinel_hip_flash_bwd_sparse(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                             out.buffer.deviceData, logSumExp.buffer.deviceData, outGradient.buffer.deviceData,
                                             queryGradient.buffer.deviceData, keyGradient.buffer.deviceData,
@@ -322,7 +353,7 @@ public:
                                             cosTable ? cosTable->buffer.deviceData : nullptr,
                                             sinTable ? sinTable->buffer.deviceData : nullptr,
                                             cosTable ? static_cast<int>(cosTable->rows) : 0, positionOffset, windowSize,
-                                            globalTokenCount, SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS,
+                                            globalTokenCount, SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS | layoutFlags,
                                             headCount, kvHeads, headDimension, static_cast<int>(query.cols), columnStart,
                                             columnCount, packCount, scale, 1, ws, wsBytes, activeStream()));
     }
@@ -345,15 +376,49 @@ private:
         return kvHeads;
     }
 
-    // Scratch for MFMA arithmetic on Sentinel's layout; one process-wide buffer that only grows (its first
-    // growth allocates, so warm it up before capturing a graph).
+    // Scratch for MFMA arithmetic on Sentinel's layout: the caller's KeptOperands where given (sized for the backward
+    // call, filled by the forward call, reused by a backward call of the same shape), else one process-wide buffer that
+    // only grows (its first growth allocates, so warm it up before capturing a graph).  `layoutFlags` comes back with
+    // the workspace flag to OR into the layout argument.
     static size_t workspaceFor(int headCount, int kvHeads, int headDimension, const HipMatrix& query, int columnStart,
-                               int columnCount, int packCount, bool backward, void*& ws) {
+                               int columnCount, int packCount, bool backward, void*& ws, KeptOperands* kept,
+                               const void* tables, int windowSize, int globalTokenCount, int positionOffset,
+                               int& layoutFlags) {
         static HipDeviceBuffer scratch;
+        layoutFlags = 0;
         const int resolved = columnCount > 0 ? columnCount : static_cast<int>(query.cols) - columnStart;
-        const size_t need = sentinel_hip_flash_workspace_bytes(SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS,
-                                                               headCount, kvHeads, headDimension, resolved > 0 ? resolved : 1,
-                                                               packCount > 0 ? packCount : 1, backward ? 1 : 0);
+        auto bytesFor = [&](bool forBackward) {
+            return sentinel_hip_flash_workspace_bytes(SENTINEL_HIP_F32, computeType(), SENTINEL_HIP_LAYOUT_COLUMNS, headCount,
+                                                      kvHeads, headDimension, resolved > 0 ? resolved : 1,
+                                                      packCount > 0 ? packCount : 1, forBackward ? 1 : 0);
+        };
+        if (kept) {
+            const int geometry[11] = {headCount,   kvHeads,       headDimension, static_cast<int>(query.cols), columnStart, columnCount,
+                                      packCount,   computeType(), windowSize,    globalTokenCount,             positionOffset};
+            const size_t keptBytes = bytesFor(true);
+            if (keptBytes == 0) {
+                kept->filled = false;  // exact fp32 arithmetic converts nothing
+            } else if (!backward) {
+                kept->workspace.ensureCapacity(keptBytes);
+                kept->filled = true;
+                kept->query = query.buffer.deviceData;
+                kept->tables = tables;
+                for (int i = 0; i < 11; ++i) kept->geometry[i] = geometry[i];
+                layoutFlags = SENTINEL_HIP_WORKSPACE_KEEP;
+                ws = kept->workspace.deviceData;
+                return keptBytes;
+            } else if (kept->filled && kept->workspace.capacityBytes >= keptBytes && kept->query == query.buffer.deviceData &&
+                       kept->tables == tables) {
+                bool same = true;
+                for (int i = 0; i < 11; ++i) same = same && kept->geometry[i] == geometry[i];
+                if (same) {
+                    layoutFlags = SENTINEL_HIP_WORKSPACE_REUSE;
+                    ws = kept->workspace.deviceData;
+                    return keptBytes;
+                }
+            }
+        }
+        const size_t need = bytesFor(backward);
         if (need == 0) return 0;
         scratch.ensureCapacity(need);
         ws = scratch.deviceData;

@@ -106,6 +106,22 @@ static void runCase(const char* name, int e, int heads, int kvHeads, int d, int 
     if (ey > tol || ex > tol || eq > tol || ek > tol || ev > tol || eo > tol) throw std::runtime_error(std::string(name) + " parity failed");
     if (layer.usedFlashAttention != preferFlash || layer.activePackCount != packs || layer.activeSegmentLength != T)
         throw std::runtime_error("layer bookkeeping");
+    if (compute != SENTINEL_HIP_COMPUTE_AUTO && preferFlash) {
+        // MFMA arithmetic: the backward call above used the 16-bit operands the forward call left behind; converting
+        // them again instead (keepFlashOperands = false) runs the same kernels on the same values
+        if (!layer.flashOperands.filled) throw std::runtime_error(std::string(name) + " forward did not keep its 16-bit operands");
+        const std::vector<float> keptDx = dx.download(), keptDwq = dwq.download(), keptDwk = dwk.download(), keptDwv = dwv.download();
+        layer.keepFlashOperands = false;
+        HipMatrix y2, dx2, a, b, c, o2;
+        layer.forward(x, y2, T);
+        layer.backward(g, dx2, a, b, c, o2);
+        if (dx2.download() != keptDx || a.download() != keptDwq || b.download() != keptDwk || c.download() != keptDwv)
+            throw std::runtime_error(std::string(name) + " kept 16-bit operands changed the gradients");
+        layer.keepFlashOperands = true;
+        layer.forward(x, y2, T);  // leave the layer as the checks below expect it: operands kept
+    } else if (layer.flashOperands.filled) {
+        throw std::runtime_error(std::string(name) + " exact fp32 arithmetic keeps no 16-bit operands");
+    }
     if (heads == kvHeads) {
         // the stacked weight gradient alone (materializeSplitWeightGrads = false) holds the same three blocks
         HipMatrix dx2, a, b, c, o2;
