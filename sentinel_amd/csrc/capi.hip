@@ -232,7 +232,7 @@ struct RopeRequest {
 const RopeRequest kNoRope = {nullptr, nullptr, 0, 0, false};
 
 int resolve_rope(const char* op, const RopeRequest& req, const Resolved& r, RopeTables* rope) {
-    *rope = RopeTables{nullptr, nullptr, 0};
+    *rope = RopeTables{nullptr, nullptr, 0, 0};
     if (!req.requested) return SENTINEL_HIP_OK;
     const int rc = check_rope(op, req.cos, req.sin, req.table_positions, r.g.head_dim, req.position_offset, r.g.seq_len);
     if (rc != SENTINEL_HIP_OK) return rc;
@@ -243,7 +243,7 @@ int resolve_rope(const char* op, const RopeRequest& req, const Resolved& r, Rope
                     "%s the rotation is fused into the layout conversion of fp32 column tensors with 16-bit arithmetic; "
                     "rotate other tensors with sentinel_hip_rope_rotate",
                     op);
-    *rope = RopeTables{req.cos, req.sin, req.position_offset};
+    *rope = RopeTables{req.cos, req.sin, req.position_offset, req.table_positions};
     return SENTINEL_HIP_OK;
 }
 
@@ -312,7 +312,7 @@ int flash_fwd(const char* op, const void* q, const void* k, const void* v, void*
     void* v16 = static_cast<char*>(k16) + kv_bytes16(g);
     const long long off = r.column_start;
     const int stride = static_cast<int>(r.stride);
-    const RopeTables none = {nullptr, nullptr, 0};
+    const RopeTables none = {nullptr, nullptr, 0, 0};
     hipError_t err = launch_columns_to_bhtd(type, static_cast<const float*>(q) + off, q16, g.q_heads, g.head_dim, stride,
                                             g.seq_len, g.packs, rope, stream);
     if (err == hipSuccess)
@@ -399,7 +399,7 @@ int flash_bwd(const char* op, const void* q, const void* k, const void* v, const
     const long long off = r.column_start;
     const int stride = static_cast<int>(r.stride);
     const int T = g.seq_len;
-    const RopeTables none = {nullptr, nullptr, 0};
+    const RopeTables none = {nullptr, nullptr, 0, 0};
     // SENTINEL_HIP_WORKSPACE_REUSE: q16, o16, k16, v16 are still the ones the forward call left there (rotated Q, K and
     // the 16-bit O the kernel itself wrote, which is the O that D = rowsum(dO o O) should be formed from anyway)
     hipError_t err = hipSuccess;

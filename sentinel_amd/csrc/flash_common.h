@@ -62,6 +62,7 @@ struct RopeTables {
     const float* cos;
     const float* sin;
     int offset;
+    int positions;  // rows of each table
 };
 
 // A result tensor in Sentinel's column layout, fp32 [(head * head_dim + dim), column], for the MFMA kernels to write
@@ -74,7 +75,7 @@ struct ColumnSink {
     long long stride;  // columns per row
     RopeTables inverse_rope;
 };
-constexpr ColumnSink kNoColumnSink = {nullptr, 0, {nullptr, nullptr, 0}};
+constexpr ColumnSink kNoColumnSink = {nullptr, 0, {nullptr, nullptr, 0, 0}};
 
 // ---- MFMA path (flash_mfma_*.hip): bf16 / fp16 [B,H,T,d] tensors, head_dim 64 or 128 ----
 bool mfma_supported(int head_dim);

@@ -43,9 +43,10 @@ __device__ __forceinline__ void store_block_to_sink(const f32x16 (&acc)[D / 32],
     float* head_rows = sink.base + (long long)head * D * sink.stride + (long long)pack * seq_len + token0;
     if (sink.inverse_rope.cos)
         store_columns_f32<D, true>(acc, factor, head_rows, (int)sink.stride, seq_len - token0, lane, sink.inverse_rope.cos,
-                                   sink.inverse_rope.sin, sink.inverse_rope.offset + token0);
+                                   sink.inverse_rope.sin, sink.inverse_rope.offset + token0,
+                                   sink.inverse_rope.positions - (sink.inverse_rope.offset + token0));
     else
-        store_columns_f32<D, false>(acc, factor, head_rows, (int)sink.stride, seq_len - token0, lane, nullptr, nullptr, 0);
+        store_columns_f32<D, false>(acc, factor, head_rows, (int)sink.stride, seq_len - token0, lane, nullptr, nullptr, 0, 0);
 }
 constexpr int kOperandLead = 4;
 

@@ -316,7 +316,7 @@ constexpr int kXcds = 8;
 template <int D, bool ROTATE>
 __device__ __forceinline__ void store_columns_f32(const f32x16 (&acc)[D / 32], float factor, float* head_rows, int stride,
                                                   int valid_rows, int lane, const float* cos_table, const float* sin_table,
-                                                  int position0) {
+                                                  int position0, int table_rows_left) {
 #pragma clang fp contract(off)
     asm volatile("" : "+v"(lane));  // keeps the per-lane address arithmetic here instead of hoisted over the caller's loops
     const int n = lane % 32;
@@ -327,11 +327,14 @@ __device__ __forceinline__ void store_columns_f32(const f32x16 (&acc)[D / 32], f
     __amdgpu_buffer_rsrc_t cos_rows = rows, sin_rows = rows;
     int table_bytes = 0;
     if (ROTATE) {
-        cos_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(cos_table) + (long long)position0 * (D / 2), 0, 0x7fffffff,
+        // the tables' rows from position0 on, with their true extent
+        const long long extent = (long long)table_rows_left * (D / 2) * 4;
+        const int records = extent > 0x7fffffffLL ? 0x7fffffff : (int)extent;
+        cos_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(cos_table) + (long long)position0 * (D / 2), 0, records,
                                                      0x00020000);
-        sin_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sin_table) + (long long)position0 * (D / 2), 0, 0x7fffffff,
+        sin_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sin_table) + (long long)position0 * (D / 2), 0, records,
                                                      0x00020000);
-        table_bytes = (n * (D / 2) + gh * 2) * 4;
+        table_bytes = n * (D / 2) * 4;
     }
 #pragma unroll
     for (int cb = 0; cb < D / 32; ++cb)
@@ -342,11 +345,12 @@ __device__ __forceinline__ void store_columns_f32(const f32x16 (&acc)[D / 32], f
 #pragma unroll
             for (int j = 0; j < 4; ++j) x[j] = acc[cb][a * 4 + j] * factor;
             if (ROTATE) {
-                // (two 32-bit loads per table: the 64-bit buffer load builtin of this toolchain fetches one word only)
-                const float c0 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cos_rows, table_bytes, (dim / 2) * 4, 0));
-                const float c1 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cos_rows, table_bytes, (dim / 2) * 4 + 4, 0));
-                const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sin_rows, table_bytes, (dim / 2) * 4, 0));
-                const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sin_rows, table_bytes, (dim / 2) * 4 + 4, 0));
+                // (one aligned 128-bit load per table = the four pairs of these eight head dims, of which a lane uses the
+                //  first or the second two: the 64-bit buffer load builtin of this toolchain fetches one word only)
+                const u32x4 cw = __builtin_amdgcn_raw_buffer_load_b128(cos_rows, table_bytes, (dim / 2) * 4, 0);
+                const u32x4 sw = __builtin_amdgcn_raw_buffer_load_b128(sin_rows, table_bytes, (dim / 2) * 4, 0);
+                const float c0 = __builtin_bit_cast(float, gh ? cw[2] : cw[0]), c1 = __builtin_bit_cast(float, gh ? cw[3] : cw[1]);
+                const float s0 = __builtin_bit_cast(float, gh ? sw[2] : sw[0]), s1 = __builtin_bit_cast(float, gh ? sw[3] : sw[1]);
                 const float e0 = x[0], o0 = x[1], e1 = x[2], o1 = x[3];
                 x[0] = e0 * c0 + o0 * s0;
                 x[1] = -e0 * s0 + o0 * c0;
