@@ -35,13 +35,18 @@ def test_rope_rotate_is_bit_identical_to_the_oracle(shape, inverse):
 
 
 @pytest.mark.parametrize("compute", ["bf16", "fp16"])
-@pytest.mark.parametrize("shape", [(4, 4, 64, 128, 1, 0, 0, 0), (8, 2, 128, 200, 2, 4, 4, 0), (2, 1, 64, 70, 3, 3, 1, 11)])
+# (q heads, kv heads, head_dim, T, packs, first column, columns behind the window, position offset, spare table rows);
+# the gradients and O are written by the attention kernels themselves, 32 tokens per store: sequence lengths around and
+# off the multiples of 32, windows that start and end inside a matrix, and tables that end exactly at the last position
+@pytest.mark.parametrize("shape", [(4, 4, 64, 128, 1, 0, 0, 0, 3), (8, 2, 128, 200, 2, 4, 4, 0, 3), (2, 1, 64, 70, 3, 3, 1, 11, 3),
+                                   (2, 1, 128, 33, 2, 5, 3, 2, 0), (4, 2, 64, 257, 1, 1, 0, 0, 0), (3, 3, 128, 31, 3, 0, 2, 9, 0),
+                                   (2, 2, 64, 1, 2, 2, 1, 0, 0)])
 def test_fused_rope_attention_matches_oracle(compute, shape):
     from sentinel_amd import HipFlashAttention
-    hq, hkv, d, t, packs, col0, pad, offset = shape
+    hq, hkv, d, t, packs, col0, pad, offset, spare = shape
     print(f"case fused rope {compute} {shape}", flush=True)
     q, k, v, g = gpu_util.make_inputs(hq, hkv, d, t, packs, seed=sum(shape) + 1, dtype=compute, col0=col0, pad=pad)
-    cos, sin = oracle_lib.rope_tables(d, t + offset + 3)
+    cos, sin = oracle_lib.rope_tables(d, t + offset + spare)
     # the oracle rotates every pack like a sequence of its own: with an offset, segment by segment
     def rotate(x, heads, inverse=False):
         y = x.copy()
