@@ -313,14 +313,13 @@ int flash_fwd(const char* op, const void* q, const void* k, const void* v, void*
     const long long off = r.column_start;
     const int stride = static_cast<int>(r.stride);
     const RopeTables none = {nullptr, nullptr, 0, 0};
-    hipError_t err = launch_columns_to_bhtd(type, static_cast<const float*>(q) + off, q16, g.q_heads, g.head_dim, stride,
-                                            g.seq_len, g.packs, rope, stream);
-    if (err == hipSuccess)
-        err = launch_columns_to_bhtd(type, static_cast<const float*>(k) + off, k16, g.kv_heads, g.head_dim, stride,
-                                     g.seq_len, g.packs, rope, stream);
-    if (err == hipSuccess)
-        err = launch_columns_to_bhtd(type, static_cast<const float*>(v) + off, v16, g.kv_heads, g.head_dim, stride,
-                                     g.seq_len, g.packs, none, stream);
+    // Q, K (rotated where the call rotates) and V in one launch
+    ConvertJobs in;
+    in.count = 3;
+    in.job[0] = ConvertJob{static_cast<const float*>(q) + off, static_cast<unsigned short*>(q16), g.q_heads, 1, 0};
+    in.job[1] = ConvertJob{static_cast<const float*>(k) + off, static_cast<unsigned short*>(k16), g.kv_heads, 1, 0};
+    in.job[2] = ConvertJob{static_cast<const float*>(v) + off, static_cast<unsigned short*>(v16), g.kv_heads, 0, 0};
+    hipError_t err = launch_columns_to_bhtd_jobs(type, in, g.head_dim, stride, g.seq_len, g.packs, rope, stream);
     // O goes to the caller's matrix straight from the kernel's accumulators (and in 16 bit to the workspace, for the
     // backward); a conversion pass only where the kernel's 32-bit row offsets would not reach
     const bool direct = direct_columns(r);
@@ -402,23 +401,17 @@ int flash_bwd(const char* op, const void* q, const void* k, const void* v, const
     const RopeTables none = {nullptr, nullptr, 0, 0};
     // SENTINEL_HIP_WORKSPACE_REUSE: q16, o16, k16, v16 are still the ones the forward call left there (rotated Q, K and
     // the 16-bit O the kernel itself wrote, which is the O that D = rowsum(dO o O) should be formed from anyway)
-    hipError_t err = hipSuccess;
+    // one launch converts dO and, unless the forward call left them, Q, K (rotated where the call rotates), V and O
+    ConvertJobs in;
+    in.count = 0;
+    in.job[in.count++] = ConvertJob{static_cast<const float*>(d_out) + off, static_cast<unsigned short*>(g16), g.q_heads, 0, 0};
     if (!r.reuse) {
-        err = launch_columns_to_bhtd(type, static_cast<const float*>(q) + off, q16, g.q_heads, g.head_dim, stride, T, g.packs,
-                                     rope, stream);
-        if (err == hipSuccess)
-            err = launch_columns_to_bhtd(type, static_cast<const float*>(out) + off, o16, g.q_heads, g.head_dim, stride, T,
-                                         g.packs, none, stream);
-        if (err == hipSuccess)
-            err = launch_columns_to_bhtd(type, static_cast<const float*>(k) + off, k16, g.kv_heads, g.head_dim, stride, T,
-                                         g.packs, rope, stream);
-        if (err == hipSuccess)
-            err = launch_columns_to_bhtd(type, static_cast<const float*>(v) + off, v16, g.kv_heads, g.head_dim, stride, T,
-                                         g.packs, none, stream);
+        in.job[in.count++] = ConvertJob{static_cast<const float*>(q) + off, static_cast<unsigned short*>(q16), g.q_heads, 1, 0};
+        in.job[in.count++] = ConvertJob{static_cast<const float*>(out) + off, static_cast<unsigned short*>(o16), g.q_heads, 0, 0};
+        in.job[in.count++] = ConvertJob{static_cast<const float*>(k) + off, static_cast<unsigned short*>(k16), g.kv_heads, 1, 0};
+        in.job[in.count++] = ConvertJob{static_cast<const float*>(v) + off, static_cast<unsigned short*>(v16), g.kv_heads, 0, 0};
     }
-    if (err == hipSuccess)
-        err = launch_columns_to_bhtd(type, static_cast<const float*>(d_out) + off, g16, g.q_heads, g.head_dim, stride, T,
-                                     g.packs, none, stream);
+    hipError_t err = launch_columns_to_bhtd_jobs(type, in, g.head_dim, stride, T, g.packs, rope, stream);
     // The gradients leave the kernels as fp32 columns, straight from the accumulators, rotated back on the way (they are
     // gradients with respect to the unrotated Q, K).  The one-pass variant and matrices beyond the kernels' 32-bit row
     // offsets write 16-bit tensors and convert them in passes of their own.

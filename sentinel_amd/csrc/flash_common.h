@@ -96,6 +96,22 @@ hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* 
 size_t bwd_stored_scratch_bytes(const AttnGeom& g);
 
 // ---- layout adapter (layout_adapter.hip): Sentinel column layout fp32 <-> [B,H,T,d] bf16 / fp16 ----
+// several tensors of one shape family (same head_dim, stride, sequence length, packs; head counts may differ) through one
+// launch; `rotate`: apply the rotary tables to this tensor; z_end is filled in by the launcher
+constexpr int kMaxConvertJobs = 5;
+struct ConvertJob {
+    const float* src;     // first column of pack 0
+    unsigned short* dst;  // [packs, heads, seq_len, head_dim]
+    int heads;
+    int rotate;
+    int z_end;
+};
+struct ConvertJobs {
+    ConvertJob job[kMaxConvertJobs];
+    int count;
+};
+hipError_t launch_columns_to_bhtd_jobs(Elem type, ConvertJobs jobs, int head_dim, int stride_columns, int seq_len, int packs,
+                                       RopeTables rope, hipStream_t stream);
 hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int heads, int head_dim, int stride_columns,
                                   int seq_len, int packs, RopeTables rope, hipStream_t stream);
 hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,

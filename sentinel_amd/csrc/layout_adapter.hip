@@ -40,14 +40,24 @@ __device__ __forceinline__ void rotate_pair(float& even, float& odd, float c, fl
 // token-major side (fp32, 4 tokens per thread) and the dim-major side (16 bit, 8 dims = 16 bytes per thread)
 // both touch 64 different banks per wavefront access.  VEC4: the fp32 rows can be accessed as aligned float4
 // (pointer, stride and sequence length all multiples of 4 floats); otherwise the same code runs on scalars.
+// Up to kMaxConvertJobs tensors of one call (Q, K, V; or Q, O, K, V, dO) go through one launch: at the sequence lengths
+// Sentinel trains with a conversion takes about as long as its launch, and three to five of them were 40 % of a step.
+// grid.z runs over the (pack, head) pairs of all jobs one after the other; z_end is the running total.
 template <typename E, bool VEC4>
-__global__ __launch_bounds__(256) void columns_to_bhtd_kernel(const float* __restrict__ src, unsigned short* __restrict__ dst,
-                                                               int heads, int d, long long stride, int T, RopeTables rope) {
+__global__ __launch_bounds__(256) void columns_to_bhtd_kernel(ConvertJobs jobs, int d, long long stride, int T, RopeTables tables) {
     __shared__ float tile[kTile][kTile + 1];
     const int t0 = blockIdx.x * kTile;
     const int c0 = blockIdx.y * kTile;
-    const int b = blockIdx.z / heads;
-    const int h = blockIdx.z % heads;
+    int job = 0, z = blockIdx.z;
+    while (job + 1 < jobs.count && (int)blockIdx.z >= jobs.job[job].z_end) ++job;
+    if (job > 0) z -= jobs.job[job - 1].z_end;
+    const float* __restrict__ src = jobs.job[job].src;
+    unsigned short* __restrict__ dst = jobs.job[job].dst;
+    const int heads = jobs.job[job].heads;
+    RopeTables rope = tables;
+    if (!jobs.job[job].rotate) rope.cos = nullptr;
+    const int b = z / heads;
+    const int h = z % heads;
     const int tid = threadIdx.x;
     {
         const int t4 = (tid % 16) * 4;
@@ -192,16 +202,32 @@ static bool rows_vec4(const void* base, int stride_columns, int seq_len) {
     return (reinterpret_cast<uintptr_t>(base) & 15u) == 0 && stride_columns % 4 == 0 && seq_len % 4 == 0;
 }
 
-hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int heads, int head_dim, int stride_columns,
-                                  int seq_len, int packs, RopeTables rope, hipStream_t stream) {
-    const dim3 grid((seq_len + kTile - 1) / kTile, (head_dim + kTile - 1) / kTile, packs * heads);
-    auto out = static_cast<unsigned short*>(dst);
-    if (head_dim % 8 != 0) return hipErrorInvalidValue;
-    const bool v4 = rows_vec4(src, stride_columns, seq_len);
+hipError_t launch_columns_to_bhtd_jobs(Elem type, ConvertJobs jobs, int head_dim, int stride_columns, int seq_len, int packs,
+                                       RopeTables rope, hipStream_t stream) {
+    if (jobs.count <= 0 || jobs.count > kMaxConvertJobs || head_dim % 8 != 0) return hipErrorInvalidValue;
+    bool v4 = true;
+    long long z = 0;
+    for (int i = 0; i < jobs.count; ++i) {
+        v4 = v4 && rows_vec4(jobs.job[i].src, stride_columns, seq_len);
+        z += (long long)packs * jobs.job[i].heads;
+        jobs.job[i].z_end = (int)z;
+    }
+    if (z > 65535) {  // more (pack, head) pairs than a grid has rows: one launch per tensor
+        for (int i = 0; i < jobs.count; ++i) {
+            ConvertJobs one;
+            one.count = 1;
+            one.job[0] = jobs.job[i];
+            if ((long long)packs * one.job[0].heads > 65535) return hipErrorInvalidValue;
+            const hipError_t err = launch_columns_to_bhtd_jobs(type, one, head_dim, stride_columns, seq_len, packs, rope, stream);
+            if (err != hipSuccess) return err;
+        }
+        return hipSuccess;
+    }
+    const dim3 grid((seq_len + kTile - 1) / kTile, (head_dim + kTile - 1) / kTile, (unsigned)z);
     KernelTimer timer("columns_to_bhtd", stream);
 #define SENTINEL_LAUNCH(E, V) \
-    hipLaunchKernelGGL((columns_to_bhtd_kernel<E, V>), grid, dim3(256), 0, stream, src, out, heads, head_dim, \
-                       (long long)stride_columns, seq_len, rope)
+    hipLaunchKernelGGL((columns_to_bhtd_kernel<E, V>), grid, dim3(256), 0, stream, jobs, head_dim, (long long)stride_columns, \
+                       seq_len, rope)
     if (type == Elem::BF16) {
         if (v4) SENTINEL_LAUNCH(Bf16, true); else SENTINEL_LAUNCH(Bf16, false);
     } else if (type == Elem::F16) {
@@ -211,6 +237,14 @@ hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int he
     }
 #undef SENTINEL_LAUNCH
     return hipGetLastError();
+}
+
+hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int heads, int head_dim, int stride_columns,
+                                  int seq_len, int packs, RopeTables rope, hipStream_t stream) {
+    ConvertJobs jobs;
+    jobs.count = 1;
+    jobs.job[0] = ConvertJob{src, static_cast<unsigned short*>(dst), heads, rope.cos != nullptr, 0};
+    return launch_columns_to_bhtd_jobs(type, jobs, head_dim, stride_columns, seq_len, packs, rope, stream);
 }
 
 hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,
