@@ -132,26 +132,16 @@ __global__ __launch_bounds__(kLanes) void fwd_f32_kernel(const float* __restrict
     }
 }
 
-// D[h][b*T + t] = sum_c out * d_out, dims in increasing order
-__global__ __launch_bounds__(128) void delta_f32_kernel(const float* __restrict__ out, const float* __restrict__ d_out,
-                                                         float* __restrict__ delta, TensorMap qm, AttnGeom g) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= g.seq_len) return;
-    const int h = blockIdx.y;
-    const int b = blockIdx.z;
-    const long long off = b * qm.pack_stride + h * qm.head_stride + t * qm.t_stride;
-    float sum = 0.0f;
-    for (int c = 0; c < g.head_dim; ++c) sum += out[off + c * qm.c_stride] * d_out[off + c * qm.c_stride];
-    delta[(long long)h * g.packs * g.seq_len + (long long)b * g.seq_len + t] = sum;
-}
-
-// dQ: one query per lane, keys streamed through LDS.
+// dQ: one query per lane, keys streamed through LDS.  Runs first: the lane holds its query's dO row anyway, so it also
+// forms D[h][b*T + t] = sum_c out * d_out (dims in increasing order, as the reference's Delta kernel sums them,
+// CudaFlashAttention.cu:576-596) and leaves it in `delta` for the dK / dV kernel: no launch of its own for that.
 template <int DP>
 __global__ __launch_bounds__(kLanes) void bwd_dq_f32_kernel(const float* __restrict__ q, const float* __restrict__ k,
-                                                             const float* __restrict__ v, const float* __restrict__ lse,
-                                                             const float* __restrict__ d_out,
-                                                             const float* __restrict__ delta, float* __restrict__ dq,
-                                                             TensorMap qm, TensorMap km, RowMap lm, AttnGeom g) {
+                                                             const float* __restrict__ v, const float* __restrict__ out,
+                                                             const float* __restrict__ lse,
+                                                             const float* __restrict__ d_out, float* __restrict__ delta,
+                                                             float* __restrict__ dq, TensorMap qm, TensorMap km, RowMap lm,
+                                                             AttnGeom g) {
     __shared__ __attribute__((aligned(16))) float ks[kKeyStage * DP];
     __shared__ __attribute__((aligned(16))) float vs[kKeyStage * DP];
 
@@ -180,7 +170,9 @@ __global__ __launch_bounds__(kLanes) void bwd_dq_f32_kernel(const float* __restr
     }
     const float c2 = g.scale * kLog2e;
     const float lse2 = lse[b * lm.pack_stride + h * lm.head_stride + qload] * kLog2e;
-    const float dl = delta[(long long)h * g.packs * T + (long long)b * T + qload];
+    float dl = 0.0f;
+    for (int c = 0; c < d; ++c) dl += out[qoff + c * qm.c_stride] * d_out[qoff + c * qm.c_stride];
+    if (qi < T) delta[(long long)h * g.packs * T + (long long)b * T + qi] = dl;
     const int kv_end = g.causal ? min(T, tile * kLanes + kLanes) : T;
     const int window_lo = g.window > 0 ? tile * kLanes - g.window + 1 : 0;
 
@@ -328,14 +320,14 @@ hipError_t run_fwd(const float* q, const float* k, const float* v, float* out, f
 }
 
 template <int DP>
-hipError_t run_bwd(const float* q, const float* k, const float* v, const float* lse, const float* d_out,
-                   const float* delta, float* dq, float* dk, float* dv, TensorMap qm, TensorMap kvm, RowMap lm, AttnGeom g,
+hipError_t run_bwd(const float* q, const float* k, const float* v, const float* out, const float* lse, const float* d_out,
+                   float* delta, float* dq, float* dk, float* dv, TensorMap qm, TensorMap kvm, RowMap lm, AttnGeom g,
                    hipStream_t stream) {
     const int tiles = (g.seq_len + kLanes - 1) / kLanes;
     hipError_t err;
     {
         KernelTimer timer("dq_f32", stream);
-        hipLaunchKernelGGL(bwd_dq_f32_kernel<DP>, dim3(tiles, g.q_heads, g.packs), dim3(kLanes), 0, stream, q, k, v, lse,
+        hipLaunchKernelGGL(bwd_dq_f32_kernel<DP>, dim3(tiles, g.q_heads, g.packs), dim3(kLanes), 0, stream, q, k, v, out, lse,
                            d_out, delta, dq, qm, kvm, lm, g);
         err = hipGetLastError();
     }
@@ -368,18 +360,10 @@ hipError_t launch_fwd_f32(const float* q, const float* k, const float* v, float*
 hipError_t launch_bwd_f32(const float* q, const float* k, const float* v, const float* out, const float* lse,
                           const float* d_out, float* dq, float* dk, float* dv, float* delta, TensorMap qm, TensorMap kvm,
                           RowMap lm, AttnGeom g, hipStream_t stream) {
-    hipError_t err;
-    {
-        KernelTimer timer("delta_f32", stream);
-        hipLaunchKernelGGL(delta_f32_kernel, dim3((g.seq_len + 127) / 128, g.q_heads, g.packs), dim3(128), 0, stream, out,
-                           d_out, delta, qm, g);
-        err = hipGetLastError();
-    }
-    if (err != hipSuccess) return err;
-    if (g.head_dim <= 16) return run_bwd<16>(q, k, v, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);
-    if (g.head_dim <= 32) return run_bwd<32>(q, k, v, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);
-    if (g.head_dim <= 64) return run_bwd<64>(q, k, v, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);
-    return run_bwd<128>(q, k, v, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);
+    if (g.head_dim <= 16) return run_bwd<16>(q, k, v, out, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);
+    if (g.head_dim <= 32) return run_bwd<32>(q, k, v, out, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);
+    if (g.head_dim <= 64) return run_bwd<64>(q, k, v, out, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);
+    return run_bwd<128>(q, k, v, out, lse, d_out, delta, dq, dk, dv, qm, kvm, lm, g, stream);
 }
 
 }  // namespace sentinel_hip
