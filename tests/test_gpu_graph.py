@@ -1,6 +1,7 @@
-"""The entry points neither allocate nor synchronise: a training step (forward + backward), a sparse-mask step and a
-decode step are captured into one HIP graph and replayed with new tensor contents; every replay must reproduce the
-eager result bit for bit (the kernels are deterministic)."""
+"""The entry points neither allocate nor synchronise: a training step (forward + backward), a sparse-mask step, a step
+through Sentinel's column layout (rotation fused, the forward's 16-bit operands kept for the backward) and a decode step
+are captured into one HIP graph and replayed with new tensor contents; every replay must reproduce the eager result bit
+for bit (the kernels are deterministic)."""
 import pytest
 import torch
 
@@ -8,7 +9,8 @@ pytestmark = pytest.mark.gpu
 
 
 def test_captured_step_replays_bit_exactly():
-    from sentinel_amd import decode_attention, flash_attention_backward, flash_attention_forward, load_library
+    from sentinel_amd import (HipFlashAttention, decode_attention, flash_attention_backward, flash_attention_forward,
+                              load_library)
     print("case graph capture", flush=True)
     torch.manual_seed(21)
     b, hq, hkv, t, d = 2, 4, 2, 640, 128
@@ -24,7 +26,23 @@ def test_captured_step_replays_bit_exactly():
     oc = torch.empty_like(qc)
     ws = torch.empty(load_library().sentinel_hip_decode_workspace_bytes(hq, 64, length) + 16, dtype=torch.uint8, device="cuda")
 
+    # the column-layout call: fp32 [(head*d + dim), packs*T] matrices inside a wider matrix, bf16 arithmetic, rotary tables
+    tc, packs, col0 = 200, 3, 8
+    cols = col0 + packs * tc + 4
+    qm, km, vm, gm = (torch.randn(h * d, cols, device="cuda") for h in (hq, hkv, hkv, hq))
+    cos, sin = torch.randn(tc + 2, d // 2, device="cuda"), torch.randn(tc + 2, d // 2, device="cuda")
+    om, lm = torch.zeros_like(qm), torch.zeros(hq, cols, device="cuda")
+    dqm, dkm, dvm = torch.zeros_like(qm), torch.zeros_like(km), torch.zeros_like(vm)
+    dm = torch.empty(hq, packs * tc, device="cuda")
+    need = load_library().sentinel_hip_flash_workspace_bytes(0, 1, 0, hq, hkv, d, tc, packs, 1)
+    wm = torch.empty(need + 16, dtype=torch.uint8, device="cuda")
+    margs = (hq, d, float(d) ** -0.5, True, col0, tc, packs)
+    mkw = dict(kv_head_count=hkv, compute="bf16", rope=(cos, sin), workspace=wm)
+
     def step():
+        HipFlashAttention.forward_multi_head(qm, km, vm, om, lm, *margs, **mkw, keep_for_backward=True)
+        HipFlashAttention.backward_multi_head(qm, km, vm, om, lm, gm, dqm, dkm, dvm, dm, *margs, **mkw,
+                                              reuse_forward_workspace=True)
         flash_attention_forward(q, k, v, out=out, lse=lse)
         flash_attention_backward(q, k, v, out, lse, g, dq=dq, dk=dk, dv=dv, delta=delta)
         flash_attention_forward(q, k, v, out=out_s, lse=lse_s, window_size=200, global_token_count=9)
@@ -32,7 +50,7 @@ def test_captured_step_replays_bit_exactly():
                                  global_token_count=9)
         decode_attention(qc, kc, vc, length, hq, 64, kv_head_count=hkv, out=oc, workspace=ws)
 
-    results = (out, lse, dq, dk, dv, out_s, lse_s, dq_s, dk_s, dv_s, oc)
+    results = (out, lse, dq, dk, dv, out_s, lse_s, dq_s, dk_s, dv_s, oc, om, lm, dqm, dkm, dvm)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -45,13 +63,17 @@ def test_captured_step_replays_bit_exactly():
     for trial in range(3):
         for x in (q, k, v, g):
             x.copy_(torch.randn(x.shape, device="cuda").bfloat16())
-        for x in (qc, kc, vc):
+        for x in (qc, kc, vc, qm, km, vm, gm):
             x.copy_(torch.randn(x.shape, device="cuda"))
         step()  # eager
         torch.cuda.synchronize()
         want = [x.clone() for x in results]
         for x in results:
             x.fill_(float("nan"))
+        for i, x in enumerate(results):  # the column-layout calls write their pack windows only: the rest stays as in `want`
+            if any(x is m for m in (om, lm, dqm, dkm, dvm)):
+                x.copy_(want[i])
+                x[:, col0:col0 + packs * tc] = float("nan")
         graph.replay()
         torch.cuda.synchronize()
         for i, (a, w) in enumerate(zip(results, want)):
