@@ -186,6 +186,12 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 
     // one trip over tile j held in (kt, vt); the next tile streams into (kt_next, vt_next) meanwhile.
     // MASKED trips compare key against query per element; the others run the bare softmax-backward arithmetic.
+    // head_dim 64 (bound by the vector ALU, registers to spare): the dP chains start from -D held in sixteen registers, which
+    // saves the subtraction per element; head_dim 128 has no registers for that and subtracts
+    constexpr bool FOLD_DELTA = D <= 64 && !WINDOW;  // (the sparse-mask variant would drop to two wavefronts per SIMD)
+    f32x16 dp_start;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dp_start[i] = FOLD_DELTA ? -dl : 0.0f;
     auto tile_trip = [&](auto masked_tag, int j, const unsigned short* kt, const unsigned short* vt, unsigned short* kt_next,
                          unsigned short* vt_next) {
         constexpr bool MASKED = decltype(masked_tag)::value;
@@ -206,10 +212,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
                 f32x16 s;
                 f32x16 dp;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    s[i] = 0.0f;
-                    dp[i] = 0.0f;
-                }
+                for (int i = 0; i < 16; ++i) s[i] = 0.0f;
                 // program order = issue order wanted within each instruction class; the interleave of the classes
                 // is laid down by the scheduling groups at the end of the half
                 u32x4 ak[KSTEPS];
@@ -221,7 +224,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) s = E::mfma(ak[ks], qf[ks], s);
 #pragma unroll
-                for (int ks = 0; ks < KSTEPS; ++ks) dp = E::mfma(av[ks], gf[ks], dp);
+                for (int ks = 0; ks < KSTEPS; ++ks) dp = E::mfma(av[ks], gf[ks], ks == 0 ? dp_start : dp);
 
                 u32x4 kt_frag[2][CB];
 #pragma unroll
@@ -248,7 +251,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned 
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int i = half * 8 + 2 * e;
-                        dsf[half][e] = E::pack2(p[i] * (dp[i] - dl), p[i + 1] * (dp[i + 1] - dl));
+                        dsf[half][e] = FOLD_DELTA ? E::pack2(p[i] * dp[i], p[i + 1] * dp[i + 1])
+                                                  : E::pack2(p[i] * (dp[i] - dl), p[i + 1] * (dp[i + 1] - dl));
                     }
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
@@ -611,7 +615,7 @@ struct DkvLds {
     unsigned short q[QT * QS];
     unsigned short g[QT * QS];
     float lse2[QT];
-    float dl[QT];
+    float dl[QT];  // -D of the stage's queries
 };
 
 // Stage ranges of one query head for a wavefront whose 32 keys start at k0w, under the causal mask and, with
@@ -788,7 +792,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
         if (tid < QT)
             st.lse2[stage_slot(row_slot)] = live ? row_val * kLog2e : __builtin_inff();  // exp2(s - inf) = 0 for padded queries
         else if (tid < 2 * QT)
-            st.dl[stage_slot(row_slot)] = live ? row_val : 0.0f;
+            st.dl[stage_slot(row_slot)] = live ? -row_val : 0.0f;  // -D: what the dP chains start from
     };
 
     // n_iter >= 1 always (the key tile's own queries)
@@ -810,16 +814,13 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
     auto softmax_backward = [&](auto masked_tag, const f32x16& s, const f32x16& dp, const DkvLds<D>& st, int qb, int q0b,
                                 u32x4 (&pf)[2], u32x4 (&dsf)[2]) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        // lse and delta of the 16 queries this lane holds, in register order (the arrays are kept in that order)
+        // lse of the 16 queries this lane holds, in register order (the array is kept in that order); dp arrives as dP - D
         float l2[16];
-        float dl[16];
 #pragma unroll
         for (int part = 0; part < 4; ++part) {
             const int base = qb * 32 + (part >> 1) * 16 + gh * 8 + (part & 1) * 4;
             const float4 a = *reinterpret_cast<const float4*>(&st.lse2[base]);
-            const float4 d4 = *reinterpret_cast<const float4*>(&st.dl[base]);
             l2[part * 4] = a.x; l2[part * 4 + 1] = a.y; l2[part * 4 + 2] = a.z; l2[part * 4 + 3] = a.w;
-            dl[part * 4] = d4.x; dl[part * 4 + 1] = d4.y; dl[part * 4 + 2] = d4.z; dl[part * 4 + 3] = d4.w;
         }
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -830,13 +831,18 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
 #pragma unroll
                 for (int w = 0; w < 2; ++w) {
                     const int i = half * 8 + 2 * e + w;
-                    float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c2, -l2[i]));
+                    // a dead pair gets exponent -inf (p = 0 exactly).  The empty asm makes the value opaque: without it the
+                    // select is compiled into a branch around the arithmetic that feeds it, per element
+                    float exponent = __builtin_fmaf(s[i], c2, -l2[i]);
                     if (MASKED) {
+                        asm("" : "+v"(exponent));
                         const int query = q0b + perm_row_of_reg(i, gh);
-                        if ((CAUSAL && key > query) || key_dead || (WINDOW && outside_window(g, query, key))) p = 0.0f;
+                        if ((CAUSAL && key > query) || key_dead || (WINDOW && outside_window(g, query, key)))
+                            exponent = -__builtin_inff();
                     }
+                    const float p = __builtin_amdgcn_exp2f(exponent);
                     p2[w] = p;
-                    ds2[w] = p * (dp[i] - dl[i]);
+                    ds2[w] = p * dp[i];
                 }
                 pf[half][e] = E::pack2(p2[0], p2[1]);
                 dsf[half][e] = E::pack2(ds2[0], ds2[1]);
@@ -852,11 +858,14 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
         f32x16 dp[2];
         u32x4 pf[2][2];
         u32x4 dsf[2][2];
-        auto scores = [&](int blk) {  // S and dP of block blk
+        auto scores = [&](int blk) {  // S and dP - D of block blk: the dP chain starts from -D of the lane's 16 queries
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                s[blk & 1][i] = 0.0f;
-                dp[blk & 1][i] = 0.0f;
+            for (int i = 0; i < 16; ++i) s[blk & 1][i] = 0.0f;
+#pragma unroll
+            for (int part = 0; part < 4; ++part) {
+                const float4 d4 = *reinterpret_cast<const float4*>(&st.dl[blk * 32 + (part >> 1) * 16 + gh * 8 + (part & 1) * 4]);
+                dp[blk & 1][part * 4] = d4.x; dp[blk & 1][part * 4 + 1] = d4.y;
+                dp[blk & 1][part * 4 + 2] = d4.z; dp[blk & 1][part * 4 + 3] = d4.w;
             }
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
