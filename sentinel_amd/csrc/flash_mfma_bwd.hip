@@ -59,7 +59,7 @@ constexpr int kDqKeyTile = 64;
 // COLUMNS: dQ goes to the caller's fp32 column matrix (dq_columns) instead of the 16-bit tensor; a compile-time switch,
 // because with the choice made at run time the 16-bit version lost 1.5 - 2 %.
 template <typename E, int D, bool CAUSAL, bool WINDOW, bool COLUMNS = false>
-__global__ __launch_bounds__(kBwdThreads, 2) void dq_mfma_kernel(const unsigned short* __restrict__ q,
+__global__ __launch_bounds__(kBwdThreads, D <= 64 ? 3 : 2) void dq_mfma_kernel(const unsigned short* __restrict__ q,
                                                                   const unsigned short* __restrict__ k,
                                                                   const unsigned short* __restrict__ v,
                                                                   const unsigned short* __restrict__ out,
