@@ -146,59 +146,70 @@ def cpu_model():
     return "unknown"
 
 
-def cpu_baseline(name, heads_sample):
-    """The CPU oracle (a restatement of the reference's OpenMP attention) timed on a bounded sample, in the two
-    ways the reference runs it: one sequence at a time with the matrix products OpenMP-parallel inside
-    ("single-call"), and one thread per sequence of the batch with serial products ("train-loop")."""
+def cpu_baseline(name, heads_sample, full=False, loop_mode=True):
+    """The CPU oracle (a restatement of the reference's OpenMP attention) timed in the two ways the reference runs it:
+    one sequence at a time with the matrix products OpenMP-parallel inside ("single-call", Math/Matrix.cpp:139-146), and
+    one thread per sequence of the batch with serial products ("train-loop", Network/LanguageModel.cpp:1109-1125).
+    full: the whole configuration (every sequence and head); otherwise a bounded sample of `heads_sample` (batch, head)
+    pairs of one sequence, with the time of the whole configuration extrapolated linearly (heads and sequences are
+    independent on the CPU path) and labelled so."""
     import numpy as np
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib
     b, hq, hkv, t, d, dtype, sigma, _ = CONFIGS[name]
     group = hq // hkv
-    heads_sample = max(group, min(hq, heads_sample) // group * group)
+    heads_sample = hq if full else max(group, min(hq, heads_sample) // group * group)
     kv_sample = heads_sample // group
+    packs_single = b if full else 1
     threads = oracle_lib.oracle().sentinel_oracle_max_threads()
     rng = np.random.default_rng(0x5E17)
 
-    def draw(packs):
-        q = (sigma * rng.standard_normal((heads_sample * d, packs * t))).astype(np.float32)
-        k = (sigma * rng.standard_normal((kv_sample * d, packs * t))).astype(np.float32)
-        v = rng.standard_normal((kv_sample * d, packs * t)).astype(np.float32)
-        g = rng.standard_normal((heads_sample * d, packs * t)).astype(np.float32)
+    def draw(heads, kv_heads, packs):
+        q = (sigma * rng.standard_normal((heads * d, packs * t))).astype(np.float32)
+        k = (sigma * rng.standard_normal((kv_heads * d, packs * t))).astype(np.float32)
+        v = rng.standard_normal((kv_heads * d, packs * t)).astype(np.float32)
+        g = rng.standard_normal((heads * d, packs * t)).astype(np.float32)
         return q, k, v, g
 
-    # single-call mode: 1 sequence x heads_sample heads
-    q, k, v, g = draw(1)
+    pair_flops = 7.0 * t * t * d  # one (batch, head) pair, causal count
+    # single-call mode: the sequences one after the other, products parallel inside
+    q, k, v, g = draw(heads_sample, kv_sample, packs_single)
     t0 = time.perf_counter()
-    oracle_lib.oracle_attention(q, k, v, g, q_heads=heads_sample, kv_heads=kv_sample, head_dim=d, seq_len=t)
+    oracle_lib.oracle_attention(q, k, v, g, q_heads=heads_sample, kv_heads=kv_sample, head_dim=d, seq_len=t,
+                                pack_count=packs_single, pack_parallel=False)
     dt = time.perf_counter() - t0
-    flops = 7.0 * heads_sample * t * t * d
-    # train-loop mode: the b sequences of the batch in parallel, one K/V head group each
-    heads_loop = group
-    heads_sample, kv_sample = heads_loop, heads_loop // group
-    q, k, v, g = draw(b)
-    t1 = time.perf_counter()
-    oracle_lib.oracle_attention(q, k, v, g, q_heads=heads_loop, kv_heads=kv_sample, head_dim=d, seq_len=t, pack_count=b,
-                                pack_parallel=True)
-    dt_loop = time.perf_counter() - t1
-    flops_loop = 7.0 * b * heads_loop * t * t * d
-    return {
-        "value": flops / dt / 1e12,
+    pairs = packs_single * heads_sample
+    report = {
+        "value": pairs * pair_flops / dt / 1e12,
         "unit": "TFLOP/s",
         "cores": threads,
         "kind": "port",
         "cpu": cpu_model(),
-        "sample": f"single-call mode: 1 sequence x {flops / (7.0 * t * t * d):.0f} of {b * hq} (batch, head) pairs of {name}, fp32, "
-                  f"forward+backward, {dt:.1f} s, gemm/softmax OpenMP-parallel inside; same causal FLOP count although the "
-                  "CPU path multiplies the full T x T",
+        "sample": ("single-call mode: " + (f"the whole configuration, {pairs} (batch, head) pairs" if full else
+                                           f"1 sequence x {heads_sample} of {b * hq} (batch, head) pairs of {name}") +
+                   f", fp32, forward+backward, {dt:.2f} s, gemm/softmax OpenMP-parallel inside; same causal FLOP count "
+                   "although the CPU path multiplies the full T x T"),
         "seconds": dt,
-        "train_loop_mode": {"value": flops_loop / dt_loop / 1e12, "unit": "TFLOP/s", "cores": min(threads, b),
-                            "seconds": dt_loop,
-                            "sample": f"{b} sequences in parallel (one thread each, serial products) x {heads_loop} heads"},
+        "whole_config_seconds": dt * (b * hq) / pairs,
+        "whole_config_seconds_is": "measured" if full else "extrapolated from the sample (pairs are independent)",
     }
+    if loop_mode:
+        # train-loop mode: the b sequences of the batch in parallel, serial products
+        heads_loop = hq if full else group
+        q, k, v, g = draw(heads_loop, heads_loop // group, b)
+        t1 = time.perf_counter()
+        oracle_lib.oracle_attention(q, k, v, g, q_heads=heads_loop, kv_heads=heads_loop // group, head_dim=d, seq_len=t,
+                                    pack_count=b, pack_parallel=True)
+        dt_loop = time.perf_counter() - t1
+        report["train_loop_mode"] = {
+            "value": b * heads_loop * pair_flops / dt_loop / 1e12, "unit": "TFLOP/s", "cores": min(threads, b),
+            "seconds": dt_loop, "whole_config_seconds": dt_loop * hq / heads_loop,
+            "whole_config_seconds_is": "measured" if full else "extrapolated from the sample (heads are independent)",
+            "sample": f"{b} sequences in parallel (one thread each, serial products) x {heads_loop} of {hq} heads"}
+    return report
 
 
-def columns_path(torch, name, steps, separate):
+def columns_path(torch, name, steps, separate, modes=None):
     """The same step through Sentinel's own tensor layout (fp32 [(head*d + dim), B*T]) with 16-bit arithmetic:
     what the drop-in costs on top of the kernels (layout / type conversion passes, optionally with the rotary
     embedding fused into them instead of four separate elementwise passes)."""
@@ -243,7 +254,8 @@ def columns_path(torch, name, steps, separate):
             HipOps.rotary_rotate_inverse_in_place(k, hkv, d, d // 2, cos, sin, 0, t)
 
     report = {}
-    modes = ("plain", "plain_kept", "fused", "fused_kept") + (("separate",) if separate else ())
+    if modes is None:
+        modes = ("plain", "plain_kept", "fused", "fused_kept") + (("separate",) if separate else ())
     for mode in modes:
         for _ in range(2):
             step(mode)
@@ -260,14 +272,10 @@ def columns_path(torch, name, steps, separate):
     times = sentinel_amd.collect_kernel_timings()
     sentinel_amd.set_kernel_timing(False)
     report["kernels_ms"] = {kname: tot / max(n, 1) for kname, (tot, n) in times.items()}
-    # conversion passes move 4 + 2 bytes per element; the in-place rotation 4 + 4
-    elems = float(hq * d) * cols
-    for kname, per_elem in (("columns_to_bhtd", 6.0), ("bhtd_to_columns", 6.0)):
+    for kname in ("columns_to_bhtd", "bhtd_to_columns"):  # conversion passes: 4 + 2 bytes per element
         if kname in times:
-            tot, n = times[kname]
-            # launches mix Q-sized and K/V-sized tensors: count the bytes of all of them
-            q_like = 3 + 1  # q, out, d_out in; dq out (+ q in, out out in the forward)
-            report[kname + "_avg_ms"] = tot / max(n, 1)
+            report[kname + "_avg_ms"] = times[kname][0] / max(times[kname][1], 1)
+    elems = float(hq * d) * cols
     flops = 7.0 * float(b) * hq * t * t * d
     for mode in modes:
         report[mode + "_tflops"] = flops / (report[mode + "_ms_per_step"] * 1e-3) / 1e12
@@ -367,6 +375,31 @@ def sparse_path(torch, name, steps):
     return report
 
 
+def profiler_attached():
+    """True under rocprofv3 (its preloaded tool library has initialised the GPU before this program started, and a
+    process that has done so must not start another program)."""
+    env = os.environ
+    return "rocprof" in env.get("LD_PRELOAD", "").lower() or any(k.startswith(("ROCPROF", "ROCP_")) for k in env)
+
+
+def layer_path(columns, steps):
+    """The attention layer behind the reference's class interface (include/sentinel_hip/HipCausalSelfAttention.hpp:
+    projections, rotation, attention core, output projection and their backward) with flash attention on and off, on
+    the reference's flash-parity shapes: the "attention fwd/bwd ms" of its train profile.  Timed by the C++ program
+    tests/cpp/bench_layer (the layer is C++), started as a child process before this process touches the GPU."""
+    import subprocess
+    exe = os.path.join(ROOT, "tests", "cpp", "bench_layer")
+    if not os.path.exists(exe):
+        return {"skipped": "tests/cpp/bench_layer is not built (python -c 'import __graft_entry__ as g; g.build()')"}
+    try:
+        proc = subprocess.run([exe, str(columns), str(steps), "3"], capture_output=True, text=True, timeout=240)
+    except (OSError, subprocess.SubprocessError) as exc:
+        return {"skipped": f"bench_layer did not run: {exc}"}
+    if proc.returncode != 0:
+        return {"skipped": f"bench_layer exit code {proc.returncode}: {proc.stderr.strip()[-300:]}"}
+    return json.loads(proc.stdout.strip().splitlines()[-1])
+
+
 def rocminfo_gpu_clock_ghz():
     """Max Clock Freq. of the first gfx agent as printed by rocminfo (GHz), 0.0 if it cannot be read."""
     import re
@@ -396,6 +429,10 @@ def main():
                          "embedding), reported under \"columns_path\"")
     ap.add_argument("--columns-separate-rope", action="store_true",
                     help="columns_path also times the reference's sequence of separate in-place rotary passes")
+    ap.add_argument("--no-layer-path", action="store_true",
+                    help="skip timing the C++ attention layer with flash attention on and off (\"layer_path\"; a child "
+                         "process, started first; skipped by itself under a profiler)")
+    ap.add_argument("--layer-columns", type=int, default=4096, help="tokens per step of the layer timing")
     ap.add_argument("--sparse-path", action="store_true",
                     help="also time the step under sliding-window + global-token masks and report it under \"sparse_path\"")
     ap.add_argument("--decode-path", action="store_true",
@@ -409,6 +446,13 @@ def main():
               "exchange, so a multi-GPU figure would be N independent copies of this one", file=sys.stderr)
         sys.exit(2)
 
+    # child processes first: nothing may be started once this process has initialised the GPU
+    layer = None
+    if not args.no_layer_path:
+        layer = ({"skipped": "a profiler is attached"} if profiler_attached()
+                 else layer_path(args.layer_columns, max(args.steps // 2, 5)))
+    fallback_clock_ghz = rocminfo_gpu_clock_ghz() if not profiler_attached() else 0.0
+
     import torch
     import sentinel_amd
     if not torch.cuda.is_available():
@@ -419,8 +463,8 @@ def main():
     props = torch.cuda.get_device_properties(0)
     cus = int(props.multi_processor_count)
     clock_ghz = float(getattr(props, "clock_rate", 0)) / 1e6  # kHz -> GHz
-    if clock_ghz <= 0.0:  # not filled in by this torch build: ask rocminfo for the GPU agent's maximum clock
-        clock_ghz = rocminfo_gpu_clock_ghz()
+    if clock_ghz <= 0.0:  # not filled in by this torch build: what rocminfo printed for the GPU agent's maximum clock
+        clock_ghz = fallback_clock_ghz
     device = {"name": props.name, "compute_units": cus, "max_clock_ghz": clock_ghz,
               # dense bf16 / fp16 MFMA: 4096 FLOP per clock per CU; the fraction below uses the published figure
               "mfma_peak_from_device_tflops": cus * 4096 * clock_ghz / 1e3}
@@ -496,6 +540,12 @@ def main():
                             "pct_of_mfma_peak": 100.0 * tf / PEAK_TFLOPS[o.dtype]}
             del o
             torch.cuda.empty_cache()
+        if "c2" in others and not args.no_columns_path:
+            # the drop-in path at the shape Sentinel itself trains with (fp32 column matrices, rotation fused, operands kept)
+            cp = columns_path(torch, "c2", 20, separate=False, modes=("fused_kept",))
+            cp["native_ms_per_step"] = others["c2"]["fwd_ms"] + others["c2"]["bwd_ms"]
+            cp["over_native"] = cp["fused_kept_ms_per_step"] / cp["native_ms_per_step"]
+            others["c2"]["columns_path"] = cp
         line["configs"] = others
 
     if not args.no_columns_path and w.dtype != "fp32":
@@ -509,8 +559,18 @@ def main():
     if args.decode_path:
         line["decode_path"] = decode_path(torch, max(args.steps, 20))
 
+    if layer is not None:
+        line["layer_path"] = layer
+
     if args.cpu_heads > 0:
         line["cpu_baseline"] = cpu_baseline(args.config, args.cpu_heads)
+        # every other configuration next to its own CPU time: C1 and C2 whole, both modes; the long ones one
+        # (batch, head) pair of one sequence in single-call mode, extrapolated
+        for name, entry in line.get("configs", {}).items():
+            entry["cpu_baseline"] = (cpu_baseline(name, 0, full=True) if name in ("c1", "c2")
+                                     else cpu_baseline(name, 1, loop_mode=False))
+            entry["speedup_over_cpu_single_call"] = (entry["cpu_baseline"]["whole_config_seconds"] /
+                                                     ((entry["fwd_ms"] + entry["bwd_ms"]) * 1e-3))
     else:
         line["cpu_baseline"] = None
     print(json.dumps(line))

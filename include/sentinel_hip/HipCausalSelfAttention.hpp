@@ -510,6 +510,9 @@ private:
     // (multi-head layers), three products otherwise (CudaCausalSelfAttention::projectAndRotate,
     // Cuda/CudaCausalSelfAttention.cu:181-208, without its three split copies)
     void project(const HipMatrix& input) {
+        // query / key / value get new contents: 16-bit copies of the old ones must not serve a later backward call (the
+        // training forward refills them right after this; prefill and decode do not)
+        flashOperands.invalidate();
         if (usesFusedQkv()) {
             syncFusedQkvWeight();
             HipGemm::multiplyInto(qkvWeight, input, qkvProjected);

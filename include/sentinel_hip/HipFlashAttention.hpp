@@ -141,13 +141,20 @@ public:
     /// backward call of the same tensors (SENTINEL_HIP_WORKSPACE_KEEP / _REUSE), the way CudaCausalSelfAttention keeps
     /// flashLogSumExp between its two calls (Cuda/CudaCausalSelfAttention.cu:237-249, :421-438): the backward call then
     /// converts outGradient only. One per layer; pass it to the forward and to the backward call. A backward call whose
-    /// shape, window, arithmetic or rotation differs from the forward call that filled it converts everything again.
+    /// matrices (query, key, value, out by device address), shape, mask, arithmetic or rotation differ from the forward
+    /// call that filled it converts everything again. What cannot be seen from here is a matrix that was overwritten in
+    /// place between the two calls: whoever does that calls invalidate().
     struct KeptOperands {
         HipDeviceBuffer workspace;
         bool filled = false;
         const void* query = nullptr;
+        const void* key = nullptr;
+        const void* value = nullptr;
+        const void* out = nullptr;
         const void* tables = nullptr;
-        int geometry[11] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        int geometry[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        /// the matrices the copies were made from have new contents: the next backward call converts them again
+        void invalidate() { filled = false; }
         void release() {
             workspace.free();
             filled = false;
@@ -171,8 +178,8 @@ public:
         logSumExp.ensureSize(static_cast<size_t>(headCount), query.cols);
         void* ws = nullptr;
         int layoutFlags = 0;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws,
-                                            kept, nullptr, 0, 0, 0, layoutFlags);
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, key, value, out, causal, columnStart, columnCount,
+                                            packCount, false, ws, kept, nullptr, 0, 0, 0, layoutFlags);
         check(sentinel_hip_flash_fwd(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                      out.buffer.deviceData, logSumExp.buffer.deviceData, SENTINEL_HIP_F32, computeType(),
                                      SENTINEL_HIP_LAYOUT_COLUMNS | layoutFlags, headCount, kvHeads, headDimension,
@@ -212,8 +219,8 @@ public:
         deltaWorkspace.ensureSize(static_cast<size_t>(headCount), static_cast<size_t>(packCount) * static_cast<size_t>(resolvedCount));
         void* ws = nullptr;
         int layoutFlags = 0;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws,
-                                            kept, nullptr, 0, 0, 0, layoutFlags);
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, key, value, out, causal, columnStart, columnCount,
+                                            packCount, true, ws, kept, nullptr, 0, 0, 0, layoutFlags);
         check(sentinel_hip_flash_bwd(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                      out.buffer.deviceData, logSumExp.buffer.deviceData, outGradient.buffer.deviceData,
                                      queryGradient.buffer.deviceData, keyGradient.buffer.deviceData,
@@ -238,8 +245,8 @@ public:
         logSumExp.ensureSize(static_cast<size_t>(headCount), query.cols);
         void* ws = nullptr;
         int layoutFlags = 0;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws,
-                                            kept, cosTable.buffer.deviceData, 0, 0, positionOffset, layoutFlags);
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, key, value, out, causal, columnStart, columnCount,
+                                            packCount, false, ws, kept, cosTable.buffer.deviceData, 0, 0, positionOffset, layoutFlags);
         check(sentinel_hip_flash_fwd_rope(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                           out.buffer.deviceData, logSumExp.buffer.deviceData, cosTable.buffer.deviceData,
                                           sinTable.buffer.deviceData, static_cast<int>(cosTable.rows), positionOffset,
@@ -274,8 +281,8 @@ public:
         deltaWorkspace.ensureSize(static_cast<size_t>(headCount), static_cast<size_t>(packCount) * static_cast<size_t>(resolvedCount));
         void* ws = nullptr;
         int layoutFlags = 0;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws,
-                                            kept, cosTable.buffer.deviceData, 0, 0, positionOffset, layoutFlags);
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, key, value, out, causal, columnStart, columnCount,
+                                            packCount, true, ws, kept, cosTable.buffer.deviceData, 0, 0, positionOffset, layoutFlags);
         check(sentinel_hip_flash_bwd_rope(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                           out.buffer.deviceData, logSumExp.buffer.deviceData, outGradient.buffer.deviceData,
                                           queryGradient.buffer.deviceData, keyGradient.buffer.deviceData,
@@ -304,8 +311,9 @@ public:
         logSumExp.ensureSize(static_cast<size_t>(headCount), query.cols);
         void* ws = nullptr;
         int layoutFlags = 0;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, false, ws,
-                                            kept, cosTable ? cosTable->buffer.deviceData : nullptr, windowSize, globalTokenCount, positionOffset, layoutFlags);
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, key, value, out, true, columnStart, columnCount,
+                                            packCount, false, ws, kept, cosTable ? cosTable->buffer.deviceData : nullptr, windowSize,
+                                            globalTokenCount, positionOffset, layoutFlags);
         check(sentinel_hip_flash_fwd_sparse(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                             out.buffer.deviceData, logSumExp.buffer.deviceData,
                                             cosTable ? cosTable->buffer.deviceData : nullptr,
@@ -344,8 +352,9 @@ public:
         deltaWorkspace.ensureSize(static_cast<size_t>(headCount), static_cast<size_t>(packCount) * static_cast<size_t>(resolvedCount));
         void* ws = nullptr;
         int layoutFlags = 0;
-        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, columnStart, columnCount, packCount, true, ws,
-                                            kept, cosTable ? cosTable->buffer.deviceData : nullptr, windowSize, globalTokenCount, positionOffset, layoutFlags);
+        const size_t wsBytes = workspaceFor(headCount, kvHeads, headDimension, query, key, value, out, true, columnStart, columnCount,
+                                            packCount, true, ws, kept, cosTable ? cosTable->buffer.deviceData : nullptr, windowSize,
+                                            globalTokenCount, positionOffset, layoutFlags);
         check(sentinel_hip_flash_bwd_sparse(query.buffer.deviceData, key.buffer.deviceData, value.buffer.deviceData,
                                             out.buffer.deviceData, logSumExp.buffer.deviceData, outGradient.buffer.deviceData,
                                             queryGradient.buffer.deviceData, keyGradient.buffer.deviceData,
@@ -380,8 +389,9 @@ private:
     // call, filled by the forward call, reused by a backward call of the same shape), else one process-wide buffer that
     // only grows (its first growth allocates, so warm it up before capturing a graph).  `layoutFlags` comes back with
     // the workspace flag to OR into the layout argument.
-    static size_t workspaceFor(int headCount, int kvHeads, int headDimension, const HipMatrix& query, int columnStart,
-                               int columnCount, int packCount, bool backward, void*& ws, KeptOperands* kept,
+    static size_t workspaceFor(int headCount, int kvHeads, int headDimension, const HipMatrix& query, const HipMatrix& key,
+                               const HipMatrix& value, const HipMatrix& out, bool causal, int columnStart, int columnCount,
+                               int packCount, bool backward, void*& ws, KeptOperands* kept,
                                const void* tables, int windowSize, int globalTokenCount, int positionOffset,
                                int& layoutFlags) {
         static HipDeviceBuffer scratch;
@@ -393,8 +403,9 @@ private:
                                                       packCount > 0 ? packCount : 1, forBackward ? 1 : 0);
         };
         if (kept) {
-            const int geometry[11] = {headCount,   kvHeads,       headDimension, static_cast<int>(query.cols), columnStart, columnCount,
-                                      packCount,   computeType(), windowSize,    globalTokenCount,             positionOffset};
+            const int geometry[12] = {headCount,   kvHeads,       headDimension, static_cast<int>(query.cols), columnStart, columnCount,
+                                      packCount,   computeType(), windowSize,    globalTokenCount,             positionOffset,
+                                      causal ? 1 : 0};
             const size_t keptBytes = bytesFor(true);
             if (keptBytes == 0) {
                 kept->filled = false;  // exact fp32 arithmetic converts nothing
@@ -402,15 +413,19 @@ private:
                 kept->workspace.ensureCapacity(keptBytes);
                 kept->filled = true;
                 kept->query = query.buffer.deviceData;
+                kept->key = key.buffer.deviceData;
+                kept->value = value.buffer.deviceData;
+                kept->out = out.buffer.deviceData;  // (the forward call has sized it before asking for the workspace)
                 kept->tables = tables;
-                for (int i = 0; i < 11; ++i) kept->geometry[i] = geometry[i];
+                for (int i = 0; i < 12; ++i) kept->geometry[i] = geometry[i];
                 layoutFlags = SENTINEL_HIP_WORKSPACE_KEEP;
                 ws = kept->workspace.deviceData;
                 return keptBytes;
             } else if (kept->filled && kept->workspace.capacityBytes >= keptBytes && kept->query == query.buffer.deviceData &&
-                       kept->tables == tables) {
+                       kept->key == key.buffer.deviceData && kept->value == value.buffer.deviceData &&
+                       kept->out == out.buffer.deviceData && kept->tables == tables) {
                 bool same = true;
-                for (int i = 0; i < 11; ++i) same = same && kept->geometry[i] == geometry[i];
+                for (int i = 0; i < 12; ++i) same = same && kept->geometry[i] == geometry[i];
                 if (same) {
                     layoutFlags = SENTINEL_HIP_WORKSPACE_REUSE;
                     ws = kept->workspace.deviceData;

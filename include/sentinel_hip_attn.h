@@ -85,18 +85,8 @@ enum { SENTINEL_HIP_LAYOUT_COLUMNS = 0, SENTINEL_HIP_LAYOUT_BHTD = 1 };
  *        mask and rotation filled, untouched since: q, k, v and out are not read or converted again, only d_out is
  *        (the q / k / v / out pointers are still validated but not dereferenced). Passing a workspace that was not
  *        filled that way gives wrong gradients: nothing can check it.
- *
- * Backward variant, OR-ed into `layout` of the backward calls (no counterpart in the reference; its backward recomputes
- * scores per tile and adds dK / dV with atomics, CudaFlashAttention.cu:1419-1425):
- *  SENTINEL_HIP_BACKWARD_STORED_SCORES  one pass over the scores: the dK / dV kernel writes the score gradients dS out
- *        in 16-bit (B * Hq * T^2 / 2 * 2 bytes in the workspace, written and read once) and dQ = scale * dS K is formed
- *        from them, instead of a second kernel recomputing S and dP. Applies to 16-bit arithmetic, head_dim 128, the
- *        plain causal mask and heads of up to 2 GiB of dS; elsewhere the flag changes nothing. The workspace grows by
- *        what sentinel_hip_flash_workspace_bytes(..., backward = 1) reports with the flag set (in the [B,H,T,d] layout
- *        that is the whole workspace). Same results as the default to rounding; measured at the
- *        same speed as the default on MI355X, which is why it is not the default.
  */
-enum { SENTINEL_HIP_WORKSPACE_KEEP = 0x100, SENTINEL_HIP_WORKSPACE_REUSE = 0x200, SENTINEL_HIP_BACKWARD_STORED_SCORES = 0x400 };
+enum { SENTINEL_HIP_WORKSPACE_KEEP = 0x100, SENTINEL_HIP_WORKSPACE_REUSE = 0x200 };
 
 /*
  * Scratch the caller must provide for a configuration (bytes; 0 when none is needed). Only the

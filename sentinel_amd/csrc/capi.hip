@@ -41,7 +41,6 @@ struct Resolved {
     bool adapter;  // column layout fp32 tensors converted to [B,H,T,d] 16-bit for the MFMA kernels
     bool keep;     // forward: lay the converted operands out where the backward expects them (SENTINEL_HIP_WORKSPACE_KEEP)
     bool reuse;    // backward: q, k, v, out of the workspace are the forward's (SENTINEL_HIP_WORKSPACE_REUSE)
-    bool stored_scores;  // backward: one pass through stored score gradients where it applies (SENTINEL_HIP_BACKWARD_STORED_SCORES)
 };
 
 // Geometry checks shared by both entry points. `op` names the operation in messages.
@@ -50,7 +49,7 @@ int resolve(const char* op, int io_dtype, int compute_dtype, int layout, int q_h
     if (io_dtype < SENTINEL_HIP_F32 || io_dtype > SENTINEL_HIP_F16) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s unknown io dtype %d", op, io_dtype);
     if (compute_dtype < SENTINEL_HIP_COMPUTE_AUTO || compute_dtype > SENTINEL_HIP_COMPUTE_F16)
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s unknown compute dtype %d", op, compute_dtype);
-    constexpr int kFlags = SENTINEL_HIP_WORKSPACE_KEEP | SENTINEL_HIP_WORKSPACE_REUSE | SENTINEL_HIP_BACKWARD_STORED_SCORES;
+    constexpr int kFlags = SENTINEL_HIP_WORKSPACE_KEEP | SENTINEL_HIP_WORKSPACE_REUSE;
     const int workspace_flags = layout & kFlags;
     layout &= ~kFlags;
     if (layout != SENTINEL_HIP_LAYOUT_COLUMNS && layout != SENTINEL_HIP_LAYOUT_BHTD)
@@ -119,7 +118,6 @@ int resolve(const char* op, int io_dtype, int compute_dtype, int layout, int q_h
     // without a conversion pass there is nothing to keep: the flags are then accepted and mean nothing
     r->keep = adapter && (workspace_flags & SENTINEL_HIP_WORKSPACE_KEEP);
     r->reuse = adapter && (workspace_flags & SENTINEL_HIP_WORKSPACE_REUSE);
-    r->stored_scores = compute != SENTINEL_HIP_COMPUTE_F32 && (workspace_flags & SENTINEL_HIP_BACKWARD_STORED_SCORES);
     return SENTINEL_HIP_OK;
 }
 
@@ -139,21 +137,18 @@ bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) !
 size_t q_bytes16(const AttnGeom& g) { return align_up((size_t)g.packs * g.q_heads * g.seq_len * g.head_dim * 2); }
 size_t kv_bytes16(const AttnGeom& g) { return align_up((size_t)g.packs * g.kv_heads * g.seq_len * g.head_dim * 2); }
 
-// 16-bit copies of the column-layout tensors (adapter), then the stored score gradients of the one-pass backward
+// 16-bit copies of the column-layout tensors (adapter)
 size_t conversion_bytes(const Resolved& r, bool backward) {
     if (!r.adapter) return 0;
     const size_t nq = q_bytes16(r.g);
     const size_t nkv = kv_bytes16(r.g);
     return backward ? 4 * nq + 4 * nkv : 2 * nq + 2 * nkv;
 }
-size_t stored_scores_bytes(const Resolved& r) { return r.stored_scores ? align_up(bwd_stored_scratch_bytes(r.g)) : 0; }
 // The kernels write fp32 column matrices with 32-bit byte offsets inside a head's rows: head_dim rows must span less
 // than 2 GiB (and likewise the rotary tables, which resolve_rope has bounded).
 bool direct_columns(const Resolved& r) { return (long long)r.g.head_dim * r.stride * 4 < 0x7fffffffLL; }
 
-size_t workspace_need(const Resolved& r, bool backward) {
-    return conversion_bytes(r, backward) + (backward ? stored_scores_bytes(r) : 0);
-}
+size_t workspace_need(const Resolved& r, bool backward) { return conversion_bytes(r, backward); }
 
 }  // namespace
 
@@ -370,13 +365,7 @@ int flash_bwd(const char* op, const void* q, const void* k, const void* v, const
         if (misaligned(q) || misaligned(k) || misaligned(v) || misaligned(out) || misaligned(d_out) || misaligned(dq) ||
             misaligned(dk) || misaligned(dv))
             return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s 16-bit tensors must be 16-byte aligned", op);
-        void* scores = nullptr;
-        if (const size_t need = stored_scores_bytes(r)) {
-            if (!workspace || workspace_bytes < need || misaligned(workspace))
-                return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s needs %zu bytes of 16-byte aligned workspace", op, need);
-            scores = workspace;
-        }
-        const hipError_t err = launch_bwd_mfma(type, q, k, v, out, lse, lse_map(r), d_out, dq, dk, dv, delta, g, stream, scores);
+        const hipError_t err = launch_bwd_mfma(type, q, k, v, out, lse, lse_map(r), d_out, dq, dk, dv, delta, g, stream);
         if (err != hipSuccess) return fail_hip("MFMA backward launch", err);
         return SENTINEL_HIP_OK;
     }
@@ -413,12 +402,11 @@ int flash_bwd(const char* op, const void* q, const void* k, const void* v, const
     }
     hipError_t err = launch_columns_to_bhtd_jobs(type, in, g.head_dim, stride, T, g.packs, rope, stream);
     // The gradients leave the kernels as fp32 columns, straight from the accumulators, rotated back on the way (they are
-    // gradients with respect to the unrotated Q, K).  The one-pass variant and matrices beyond the kernels' 32-bit row
-    // offsets write 16-bit tensors and convert them in passes of their own.
-    void* scores = stored_scores_bytes(r) ? ws + conversion_bytes(r, true) : nullptr;
-    if (!scores && direct_columns(r)) {
+    // gradients with respect to the unrotated Q, K).  Matrices beyond the kernels' 32-bit row offsets write 16-bit
+    // tensors and convert them in passes of their own.
+    if (direct_columns(r)) {
         if (err == hipSuccess)
-            err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream, nullptr,
+            err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream,
                                   ColumnSink{static_cast<float*>(dq) + off, r.stride, rope},
                                   ColumnSink{static_cast<float*>(dk) + off, r.stride, rope},
                                   ColumnSink{static_cast<float*>(dv) + off, r.stride, none});
@@ -426,7 +414,7 @@ int flash_bwd(const char* op, const void* q, const void* k, const void* v, const
         return SENTINEL_HIP_OK;
     }
     if (err == hipSuccess)
-        err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream, scores);
+        err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream);
     if (err == hipSuccess)
         err = launch_bhtd_to_columns(type, dq16, static_cast<float*>(dq) + off, g.q_heads, g.head_dim, stride, T, g.packs,
                                      rope, stream);

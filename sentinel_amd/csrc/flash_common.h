@@ -83,17 +83,12 @@ bool mfma_supported(int head_dim);
 // out_columns: O is written there as well (the 16-bit `out` is always written: the backward reads it)
 hipError_t launch_fwd_mfma(Elem type, const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm,
                            AttnGeom g, hipStream_t stream, ColumnSink out_columns = kNoColumnSink);
-// ds_scratch: bwd_stored_scratch_bytes(g) bytes for the one-pass backward (dS written by the dK / dV kernel, dQ formed
-// from it), or nullptr for the two-pass backward that recomputes S and dP in a dQ kernel of its own.
 // dq_columns / dk_columns / dv_columns: where given, that gradient goes there instead of to its 16-bit tensor (which may
-// then be nullptr); the one-pass backward does not take them.
+// then be nullptr).
 hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* v, const void* out, const float* lse,
                            RowMap lm, const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g,
-                           hipStream_t stream, void* ds_scratch = nullptr, ColumnSink dq_columns = kNoColumnSink,
+                           hipStream_t stream, ColumnSink dq_columns = kNoColumnSink,
                            ColumnSink dk_columns = kNoColumnSink, ColumnSink dv_columns = kNoColumnSink);
-// 0 where the one-pass backward does not apply (head_dim other than 128, no causal mask, sparse mask, a head's blocks
-// beyond 2 GiB)
-size_t bwd_stored_scratch_bytes(const AttnGeom& g);
 
 // ---- layout adapter (layout_adapter.hip): Sentinel column layout fp32 <-> [B,H,T,d] bf16 / fp16 ----
 // several tensors of one shape family (same head_dim, stride, sequence length, packs; head counts may differ) through one

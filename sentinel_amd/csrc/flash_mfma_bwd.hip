@@ -336,250 +336,6 @@ constexpr int kDkvQueryTile = 64;
 // ------------------------------------------------------------------------------------------------
 constexpr int kDkvSplitThreads = 512;
 
-// ------------------------------------------------------------------------------------------------
-// Stored score gradients (one-pass backward): the key-outer kernel forms dS = P o (dP - D) for every (128-key tile,
-// 64-query stage) it visits anyway; instead of recomputing S and dP in a query-outer pass (2 of that pass's 3 matrix
-// products), it writes dS out in 16-bit and a streaming kernel forms dQ = scale * dS K from it.  Trades 2U of matrix work
-// and its softmax arithmetic for B*Hq*T^2/2 * 2 bytes written and read once (HBM has the room: the MFMA kernels use about
-// an eighth of it).
-// Layout: one block of 128 keys x 64 queries (16 KiB) per (query head, key tile, stage), row = key, 64 query positions
-// per row; a head's blocks are ordered by key tile, then stage (under the causal mask only the stages from the tile's
-// diagonal on exist).  Inside a row the queries of each group of 16 sit in operand order: position 8 g + j holds query
-// 2 g + rho(j), rho = {0,4,8,12,1,5,9,13}, which is how a lane of the grad wavefront holds them (16 bytes per lane and
-// 16-query half, no shuffle before the store); the reader undoes it when it stores its result rows.
-// ------------------------------------------------------------------------------------------------
-struct DsBlocks {
-    static constexpr int kElems = kDkvKeyTile * kDkvQueryTile;  // 16-bit elements per block
-    int stages;    // 64-query stages of a sequence
-    int key_tiles;
-    int causal;
-    long long per_head;
-    static __host__ __device__ DsBlocks of(int seq_len, bool causal) {
-        DsBlocks d;
-        d.stages = (seq_len + kDkvQueryTile - 1) / kDkvQueryTile;
-        d.key_tiles = (seq_len + kDkvKeyTile - 1) / kDkvKeyTile;
-        d.causal = causal;
-        d.per_head = d.first_of_key_tile(d.key_tiles);
-        return d;
-    }
-    // key tile kt meets the stages from 2 kt on (causal) or all of them
-    __host__ __device__ long long first_of_key_tile(int kt) const {
-        return causal ? (long long)kt * stages - (long long)kt * (kt - 1) : (long long)kt * stages;
-    }
-};
-
-// D = rowsum(dO o O) for the one-pass backward (the two-pass version forms it in the dQ kernel's prologue).
-// One row of D elements per D / 8 lanes, 16 bytes of each tensor per lane.
-template <typename E, int D>
-__global__ __launch_bounds__(256) void delta_rows_kernel(const unsigned short* __restrict__ out,
-                                                         const unsigned short* __restrict__ d_out, float* __restrict__ delta,
-                                                         int q_heads, int seq_len, int packs) {
-    constexpr int LANES = D / 8;
-    const long long rows = (long long)packs * q_heads * seq_len;
-    const long long row = (long long)blockIdx.x * (256 / LANES) + threadIdx.x / LANES;
-    const int piece = threadIdx.x % LANES;
-    float sum = 0.0f;
-    if (row < rows) {
-        const u32x4 o = *reinterpret_cast<const u32x4*>(out + row * D + piece * 8);
-        const u32x4 g = *reinterpret_cast<const u32x4*>(d_out + row * D + piece * 8);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) sum += E::lo(o[e]) * E::lo(g[e]) + E::hi(o[e]) * E::hi(g[e]);
-    }
-#pragma unroll
-    for (int step = LANES / 2; step >= 1; step >>= 1) sum += __shfl_xor(sum, step);
-    if (row < rows && piece == 0) {
-        const long long t = row % seq_len;
-        const long long bh = row / seq_len;
-        const long long h = bh % q_heads, b = bh / q_heads;
-        delta[h * packs * seq_len + b * seq_len + t] = sum;
-    }
-}
-
-// 64 keys x 128 query positions of dS -> LDS (rows of the tile are 64 positions long in memory, see dq_from_ds_kernel)
-typedef DirectTile<64, 128, kBwdThreads> DqsTile;
-__device__ __forceinline__ void issue_ds_piece(__amdgpu_buffer_rsrc_t rsrc, unsigned short* stage, int thread_offset,
-                                               int piece_bytes, int wave) {
-    typedef DqsTile Tile;
-    typedef __attribute__((address_space(3))) void* lds_void;
-#pragma unroll
-    for (int it = 0; it < Tile::kIters; ++it)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void)(stage + (it * kBwdThreads + wave * 64) * 8), 16,
-                                                 thread_offset + it * Tile::kRowsPerIter * kDkvQueryTile * 2, piece_bytes, 0, 0);
-}
-
-// dQ = scale * dS K from the stored score gradients.  A workgroup of four wavefronts owns 256 queries (four stages) and
-// streams, 64 keys at a time, the K tile and the matching 64 x 256 piece of dS (64 rows of four neighbouring blocks, kept
-// as two tiles of 128 query positions) straight into LDS; both operands of dQ^T[d, q] += K^T[d, key] dS^T[key, q] contract
-// over the rows of their tile and are read with the transposing LDS reads.  A wavefront forms 64 head dims x 128 queries
-// (eight accumulator blocks): every K^T operand it reads serves four products and every dS^T operand two, 0.75 operand
-// reads per matrix instruction, which keeps the LDS (the limit of a first version with 32 queries per wavefront, 1.25
-// reads per instruction) below the one read of dS from HBM that bounds the kernel.  No softmax arithmetic.
-constexpr int kDqsQueryTile = 256;
-constexpr int kDqsKeyTile = 64;
-constexpr int kDqsStages = 3;
-template <typename E, int D, bool CAUSAL>
-__global__ __launch_bounds__(kBwdThreads, 1) void dq_from_ds_kernel(const unsigned short* __restrict__ k,
-                                                                    const unsigned short* __restrict__ ds,
-                                                                    unsigned short* __restrict__ dq, AttnGeom g, int q_tiles,
-                                                                    int total_tiles, int tiles_per_xcd) {
-    static_assert(D == 128, "a row of a dS tile and a row of K are both 128 elements");
-    constexpr int KT = kDqsKeyTile;
-    typedef DqsTile Tile;
-    static_assert(KT == 64, "DqsTile");
-    // three stages of (K tile, left dS tile, right dS tile): the loads of two trips are in flight while a third is
-    // multiplied (a request takes about 3 us under this load: what is in flight per compute unit sets the rate).  One
-    // array per stage and operand, so that requests streaming into one are known not to alias the reads of another (with
-    // one array indexed by stage the compiler waits for every request before every LDS read).
-    // (one array per stage, K | left dS | right dS: the compiler tells the targets of at most eight request sites apart,
-    //  and every unrolled copy of a trip counts)
-    __shared__ __attribute__((aligned(16))) unsigned short lds0[3 * Tile::kElems];
-    __shared__ __attribute__((aligned(16))) unsigned short lds1[3 * Tile::kElems];
-    __shared__ __attribute__((aligned(16))) unsigned short lds2[3 * Tile::kElems];
-    static_assert(4 * Tile::kElems == kDqsQueryTile * D, "the result tile leaves through two of the dS stage arrays");
-    static_assert(Tile::kIters == 4, "the partial waits below count 12 requests per trip and thread");
-
-    const int T = g.seq_len;
-    const int tid = threadIdx.x;
-    const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
-    const int wm = wave & 1;   // head dims [64 wm, 64 wm + 64)
-    const int wn = wave >> 1;  // query positions [128 wn, 128 wn + 128) of the tile
-    const int lane = tid % 64;
-    const DsBlocks blocks = DsBlocks::of(T, CAUSAL);
-
-    const int xcd = (int)blockIdx.x % kXcds;
-    const int local_tile = (int)blockIdx.x / kXcds;
-    const int tile_id = xcd * tiles_per_xcd + local_tile;
-    if (local_tile >= tiles_per_xcd || tile_id >= total_tiles) return;
-    const int bh = tile_id / q_tiles;
-    const int qt = q_tiles - 1 - tile_id % q_tiles;  // longest first within a head
-    const int b = bh / g.q_heads;
-    const int h = bh % g.q_heads;
-    const int kvh = h / (g.q_heads / g.kv_heads);
-
-    const unsigned short* kb = k + ((long long)b * g.kv_heads + kvh) * T * D;
-    const unsigned short* dsb = ds + (long long)bh * blocks.per_head * DsBlocks::kElems;
-    // keys met by the tile, and by each 128-query half of it (under the causal mask the left half stops a key tile early:
-    // the blocks of the last key tile's stages before its diagonal do not exist)
-    auto trips_below = [&](int q_end) { return CAUSAL ? (min(T, q_end) + KT - 1) / KT : (T + KT - 1) / KT; };
-    const int n_trips = trips_below((qt + 1) * kDqsQueryTile);
-    const int n_trips_left = trips_below(qt * kDqsQueryTile + 128);
-    const int my_trips = wn ? n_trips : n_trips_left;
-
-    const __amdgpu_buffer_rsrc_t k_rsrc = make_head_rsrc(kb, (long long)T * D * 2);
-    const __amdgpu_buffer_rsrc_t s_rsrc = make_head_rsrc(dsb, blocks.per_head * DsBlocks::kElems * 2);
-    const int k_off = Tile::global_offset(tid);
-    // dS tile: LDS row r (a key), 16-byte position pos holds chunk c = pos ^ (r & 15) of its 128 query positions: chunks
-    // 0..7 come from the block of the tile's first stage, 8..15 from the next block
-    int s_off;
-    {
-        const int row = tid / Tile::kChunksPerRow;
-        const int c = (tid % Tile::kChunksPerRow) ^ (row & Tile::kMask);
-        s_off = ((c >> 3) * DsBlocks::kElems + row * kDkvQueryTile + (c & 7) * 8) * 2;
-    }
-    // trip j: keys [64 j, 64 j + 64) = half j % 2 of key tile j / 2; the left dS tile holds stages 4 qt, 4 qt + 1 of
-    // that key tile, the right one stages 4 qt + 2, 4 qt + 3
-    auto issue_trip = [&](unsigned short* k_to, int j) __attribute__((always_inline)) {
-        unsigned short* s_to = k_to + Tile::kElems;
-        Tile::issue(k_rsrc, k_to, k_off, j * KT * D * 2, wave);
-        const int kt = j >> 1;
-        const long long first = blocks.first_of_key_tile(kt) + (4 * qt - (CAUSAL ? 2 * kt : 0));
-        const int row_bytes = (j & 1) * KT * kDkvQueryTile * 2;
-        // past the left half's last trip its blocks do not exist: the right half's are fetched twice (never read) so that
-        // every trip issues the same number of requests
-        const long long left = j < n_trips_left ? first : first + 2;
-        issue_ds_piece(s_rsrc, s_to, s_off, (int)(left * DsBlocks::kElems * 2) + row_bytes, wave);
-        issue_ds_piece(s_rsrc, s_to + Tile::kElems, s_off, (int)((first + 2) * DsBlocks::kElems * 2) + row_bytes, wave);
-    };
-    // (requests past the last trip repeat the last trip's: every trip then issues and waits for the same number, which
-    //  keeps the loop free of branches around the waits)
-    issue_trip(lds0, 0);
-    issue_trip(lds1, min(1, n_trips - 1));
-
-    f32x16 acc[2][4];
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[c][nb][i] = 0.0f;
-    const int t_even = Tile::transposed_read_base(lane, 0);
-    const int t_odd = Tile::transposed_read_base(lane, 1);
-    __builtin_amdgcn_s_waitcnt(0x0F7C);  // vmcnt(12): trip 0 has landed (requests complete in order)
-    __builtin_amdgcn_s_barrier();
-
-    // one trip over the tiles in (k_cur, s_cur); trip j + 2 streams into the stage trip j - 1 was read from (every
-    // wavefront has passed that trip's barrier)
-    auto tile_trip = [&](int j, const unsigned short* k_cur, unsigned short* k_to) __attribute__((always_inline)) {
-        issue_trip(k_to, min(j + 2, n_trips - 1));
-        if (j < my_trips) {
-            const unsigned short* s_mine = k_cur + (1 + wn) * Tile::kElems;
-#pragma unroll
-            for (int c4 = 0; c4 < KT / 16; ++c4) {
-                u32x4 kfrag[2], sfrag[4];
-#pragma unroll
-                for (int c = 0; c < 2; ++c)
-                    kfrag[c] = lds_read_transposed_pair(k_cur + c4 * 16 * D + (t_even ^ ((wm * 2 + c) << 5)),
-                                                        k_cur + c4 * 16 * D + (t_odd ^ ((wm * 2 + c) << 5)));
-#pragma unroll
-                for (int nb = 0; nb < 4; ++nb)
-                    sfrag[nb] = lds_read_transposed_pair(s_mine + c4 * 16 * D + (t_even ^ (nb << 5)),
-                                                         s_mine + c4 * 16 * D + (t_odd ^ (nb << 5)));
-#pragma unroll
-                for (int c = 0; c < 2; ++c)
-#pragma unroll
-                    for (int nb = 0; nb < 4; ++nb) acc[c][nb] = E::mfma(kfrag[c], sfrag[nb], acc[c][nb]);
-            }
-        }
-        // this thread's share of trip j + 1 is in LDS; trip j + 2 may still be on its way
-        __builtin_amdgcn_s_waitcnt(0x0F7C);  // vmcnt(12)
-        __builtin_amdgcn_s_barrier();
-    };
-    for (int j = 0; j < n_trips; j += 3) {  // (up to two idle trips at the end)
-        tile_trip(j, lds0, lds2);
-        tile_trip(j + 1, lds1, lds0);
-        tile_trip(j + 2, lds2, lds1);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the repeated requests of the last trips have landed too
-    __syncthreads();
-
-    // Result tile [256 query positions][128 head dims] through LDS (every stage is free: the last trip ended with a
-    // barrier): rows [0, 128) pass through lds0, rows [128, 256) through lds1.  acc[c][nb]: lane
-    // (n, gh) holds position 128 wn + 32 nb + n, head dims 64 wm + 32 c + 8 a + 4 gh + [0, 4) in registers 4 a ..; 16-byte
-    // pieces of a row are XOR-swizzled with the row number against bank conflicts.
-    {
-        const int n = lane % 32, gh = lane / 32;
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-            unsigned char* tile = reinterpret_cast<unsigned char*>(wn ? lds1 : lds0);
-            const int row = nb * 32 + n;
-#pragma unroll
-            for (int c = 0; c < 2; ++c)
-#pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    u32x2 w;
-                    w[0] = E::pack2(acc[c][nb][a * 4 + 0] * g.scale, acc[c][nb][a * 4 + 1] * g.scale);
-                    w[1] = E::pack2(acc[c][nb][a * 4 + 2] * g.scale, acc[c][nb][a * 4 + 3] * g.scale);
-                    const int piece = wm * 8 + c * 4 + a;
-                    *reinterpret_cast<u32x2*>(tile + row * (D * 2) + ((piece ^ (row & 15)) << 4) + gh * 8) = w;
-                }
-        }
-        __syncthreads();
-        // positions map back to queries: inside a group of 16, position 8 g + j is query 2 g + rho(j) (see DsBlocks)
-        unsigned short* dst = dq + (long long)bh * T * D;
-        const int p = tid % 16;
-#pragma unroll
-        for (int pass = 0; pass < kDqsQueryTile / 16; ++pass) {
-            const unsigned char* tile = reinterpret_cast<const unsigned char*>(pass < 8 ? lds0 : lds1);
-            const int r = (pass % 8) * 16 + tid / 16;  // row inside the array; same low four bits as the position
-            const u32x4 val = *reinterpret_cast<const u32x4*>(tile + r * (D * 2) + ((p ^ (r & 15)) << 4));
-            const int position = pass * 16 + tid / 16;
-            const int query = qt * kDqsQueryTile +
-                              ((position & ~15) | (((position >> 3) & 1) << 1) | ((position & 3) << 2) | ((position >> 2) & 1));
-            if (query < T) *reinterpret_cast<u32x4*>(dst + (long long)query * D + p * 8) = val;
-        }
-    }
-}
-
 template <int D>
 struct DkvSplitStage {
     static constexpr int QT = kDkvQueryTile;
@@ -936,14 +692,12 @@ __global__ __launch_bounds__(kBwdThreads, 2) void dkdv_mfma_kernel(
 }
 
 // COLUMNS: as in dkdv_mfma_kernel
-template <typename E, int D, bool CAUSAL, bool WINDOW, bool STORE_DS = false, bool COLUMNS = false>
+template <typename E, int D, bool CAUSAL, bool WINDOW, bool COLUMNS = false>
 __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     const unsigned short* __restrict__ q, const unsigned short* __restrict__ k, const unsigned short* __restrict__ v,
     const unsigned short* __restrict__ d_out, const float* __restrict__ lse, const float* __restrict__ delta,
     unsigned short* __restrict__ dk, unsigned short* __restrict__ dv, RowMap lm, AttnGeom g, int k_tiles,
-    int total_tiles, int tiles_per_xcd, int deal, unsigned short* __restrict__ ds_out, ColumnSink dk_columns,
-    ColumnSink dv_columns) {
-    static_assert(!(STORE_DS && WINDOW), "the stored score gradients cover the full causal / full rectangle only");
+    int total_tiles, int tiles_per_xcd, int deal, ColumnSink dk_columns, ColumnSink dv_columns) {
     constexpr int QT = kDkvQueryTile;
     // the query / dO tiles of a stage are staged by the score wavefronts alone (threads 0..255): they have about a
     // quarter of a stage to spare, the grad wavefronts are the critical path
@@ -1112,47 +866,6 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         __syncthreads();
     };
 
-    // Stored score gradients (STORE_DS).  The grad wavefront leaves dS of a stage in the P panels it was made from; the
-    // score wavefront of the same 32 keys, which has time to spare, copies it to memory two trips later, just before it
-    // refills that P buffer: four 128-bit reads that gather whole rows (a key's 64 query positions = 128 bytes, 8 lanes)
-    // and four stores of 1 KiB of consecutive addresses each.  ds_slot(key, panel, half g) = 32 g + (perm(key) ^ (2 panel + g))
-    // with perm(key) = key ^ ((key & 1) << 3) is the slot, inside panel (block, 16-query half), of the 16 bytes lane
-    // (key, g) holds: the XOR terms spread the 16 lanes the LDS serves together over all banks, for the row-wise reads
-    // (2 keys x 8 pieces) as well as for the writes (16 keys of one piece).
-    const int ds_key_slot = gh * 32 + ((n ^ ((n & 1) << 3)) ^ gh);  // grad lanes: slot in panel p = ds_key_slot ^ 2p
-    const int ds_write_lane = kPBase + kblock * (2 * 2 * 64 * 16);
-    int ds_read_lane = 0;          // score lanes: byte offset of the piece read by the first of the four row reads
-    unsigned short* ds_flush_at = nullptr;  // this lane's 16 bytes in the block of the next stage to be copied out
-    long long ds_next_head = 0;
-    int ds_stage_in_head = 0;
-    if constexpr (STORE_DS) {
-        const int key_lo = lane / 8, piece = lane % 8;  // row read i covers keys 8 i + key_lo, pieces (panel, g) = (piece / 2, piece % 2)
-        const int slot0 = (piece & 1) * 32 + ((key_lo ^ ((key_lo & 1) << 3)) ^ piece);  // 2 panel + g = piece
-        ds_read_lane = kPBase + kblock * (2 * 2 * 64 * 16) + (piece >> 1) * (64 * 16) + slot0 * 16;
-        const DsBlocks blocks = DsBlocks::of(T, CAUSAL);
-        ds_flush_at = ds_out +
-                      (((long long)b * g.q_heads + kvh * group) * blocks.per_head + blocks.first_of_key_tile(ktile)) *
-                          DsBlocks::kElems +
-                      kblock * 32 * kDkvQueryTile + lane * 8;
-        ds_next_head = (long long)(blocks.per_head - n_qt) * DsBlocks::kElems;
-    }
-    // copies dS of the oldest stage not yet in memory out of P buffer `buffer` (score role)
-    auto flush_ds = [&](int buffer) {
-        u32x4 rows[4];
-        const int at = opaque(ds_read_lane);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) rows[i] = *reinterpret_cast<const u32x4*>(dkv_smem + ((at ^ (i << 7)) + buffer * kPBufBytes));
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            __builtin_nontemporal_store(rows[i], reinterpret_cast<u32x4*>(ds_flush_at + i * 8 * kDkvQueryTile));
-        }
-        ds_flush_at += DsBlocks::kElems;
-        if (++ds_stage_in_head == n_qt) {  // the heads of a group are consecutive, a head's stages consecutive blocks
-            ds_stage_in_head = 0;
-            ds_flush_at += ds_next_head;
-        }
-    };
-
     // score role, trip `it`: P of both 32-query blocks of stage `it` -> LDS, dV^T += dO^T P
     auto score_trip = [&](auto masked_tag, int it) {
         constexpr bool MASKED = decltype(masked_tag)::value;
@@ -1164,9 +877,6 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         u32x4* pout = reinterpret_cast<u32x4*>(dkv_smem + opaque(p_lane + (it & 1) * kPBufBytes));
         // key - query of register i, block blk is mask_rel - (32 blk + row of register i in lane half 0): one
         // per-lane value compared against compile-time constants; a key past the end masks everything
-        if constexpr (STORE_DS) {
-            if (it >= 2) flush_ds(it & 1);  // dS of stage it - 2 leaves the buffer this trip's P goes into
-        }
         const int mask_rel = key_dead ? 0x7fffffff : (CAUSAL ? key - q0 - gh * 2 : -0x7fffffff);
         // sparse mask: a key outside the global range is dead for queries window or more behind it, i.e. from
         // 32 blk + row = mask_rel + window on
@@ -1252,13 +962,6 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
                 dsf[0][e] = E::pack2(E::lo(pf0[e]) * dp[2 * e], E::hi(pf0[e]) * dp[2 * e + 1]);
                 dsf[1][e] = E::pack2(E::lo(pf1[e]) * dp[8 + 2 * e], E::hi(pf1[e]) * dp[8 + 2 * e + 1]);
             }
-            if constexpr (STORE_DS) {
-                // dS takes the place of the P panels it was made from (every lane of this wavefront has read them), in
-                // the slot order the score wavefront's row-wise read-back wants (ds_slot)
-                unsigned char* panel = dkv_smem + opaque(ds_write_lane + ((it - 1) & 1) * kPBufBytes);
-                *reinterpret_cast<u32x4*>(panel + ((blk * 2 + 0) * 64 * 16) + (((ds_key_slot ^ (2 * (blk * 2 + 0))) << 4))) = dsf[0];
-                *reinterpret_cast<u32x4*>(panel + ((blk * 2 + 1) * 64 * 16) + (((ds_key_slot ^ (2 * (blk * 2 + 1))) << 4))) = dsf[1];
-            }
             auto dk_chain = [&] {
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
@@ -1294,9 +997,6 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
         // store dV meanwhile.  The stage buffers are still in use; the rows pass through the P buffer this trip would
         // have filled, 4 KB per wavefront, 16 rows at a time.
         static_assert(kPBufBytes >= 4 * 16 * D * 2, "P buffer too small to stage the dV rows");
-        if constexpr (STORE_DS) {
-            if (n_iter >= 2) flush_ds(n_iter & 1);  // dS of the last stage but one still sits in that buffer
-        }
         if constexpr (COLUMNS)
             store_block_to_sink<D>(acc, 1.0f, dv_columns, kvh, b, k0w, T, lane);
         else
@@ -1304,7 +1004,6 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
                 acc, 1.0f, reinterpret_cast<unsigned short*>(dkv_smem + kPBase + (n_iter & 1) * kPBufBytes) + kblock * (16 * D),
                 dv + kv_head + (long long)k0w * D, T - k0w, lane);
         __syncthreads();
-        if constexpr (STORE_DS) flush_ds((n_iter - 1) & 1);  // the last stage's dS, complete with this barrier
     } else {
         __syncthreads();  // trip 0: the score wavefronts work on stage 0 and publish stage 1
         for (int it = 1; it <= n_iter; ++it) grad_trip(it);
@@ -1323,56 +1022,9 @@ __global__ __launch_bounds__(kDkvSplitThreads) void dkdv_split_kernel(
     }  // next key tile of this workgroup (both roles have passed the last barrier of the tile: the LDS is free)
 }
 
-// one-pass backward through stored score gradients (head_dim 128, no sparse mask): D, then dK / dV with dS written out,
-// then dQ from dS
-template <typename E, int D>
-hipError_t run_bwd_stored(const unsigned short* qp, const unsigned short* kp, const unsigned short* vp, const unsigned short* op,
-                          const float* lse, RowMap lm, const unsigned short* gp, unsigned short* dqp, unsigned short* dkp,
-                          unsigned short* dvp, float* delta, AttnGeom g, unsigned short* ds, hipStream_t stream) {
-    const int T = g.seq_len;
-    {
-        const long long rows = (long long)g.packs * g.q_heads * T;
-        const int rows_per_block = 256 / (D / 8);
-        KernelTimer timer("delta_rows", stream);
-        hipLaunchKernelGGL((delta_rows_kernel<E, D>), dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0,
-                           stream, op, gp, delta, g.q_heads, T, g.packs);
-        const hipError_t err = hipGetLastError();
-        if (err != hipSuccess) return err;
-    }
-    {
-        const int k_tiles = (T + kDkvKeyTile - 1) / kDkvKeyTile;
-        const int total = g.packs * g.kv_heads * k_tiles;
-        const int tiles_per_xcd = (total + kXcds - 1) / kXcds;
-        const size_t smem = sizeof(DkvSplitLds<D>);
-        auto launch = [&](auto kernel) -> hipError_t {
-            static const hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-            if (raised != hipSuccess) return raised;
-            static const int resident = resident_workgroups_per_xcd(kernel, kDkvSplitThreads, smem);
-            const int grid = kXcds * (tiles_per_xcd < resident ? tiles_per_xcd : resident);
-            KernelTimer timer("dkdv_mfma", stream);
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp, dvp, lm, g,
-                               k_tiles, total, tiles_per_xcd, 0, ds, kNoColumnSink, kNoColumnSink);
-            return hipGetLastError();
-        };
-        const hipError_t err = launch(dkdv_split_kernel<E, D, true, false, true>);
-        if (err != hipSuccess) return err;
-    }
-    const int q_tiles = (T + kDqsQueryTile - 1) / kDqsQueryTile;
-    const int total = g.packs * g.q_heads * q_tiles;
-    const int tiles_per_xcd = (total + kXcds - 1) / kXcds;
-    auto launch = [&](auto kernel) -> hipError_t {
-        KernelTimer timer("dq_from_ds", stream);
-        hipLaunchKernelGGL(kernel, dim3(kXcds * tiles_per_xcd), dim3(kBwdThreads), 0, stream, kp, ds, dqp, g, q_tiles, total,
-                           tiles_per_xcd);
-        return hipGetLastError();
-    };
-    return launch(dq_from_ds_kernel<E, D, true>);
-}
-
 template <typename E, int D>
 hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse, RowMap lm,
-                   const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g, void* ds_scratch,
+                   const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g,
                    hipStream_t stream, ColumnSink dq_columns, ColumnSink dk_columns, ColumnSink dv_columns) {
     auto qp = static_cast<const unsigned short*>(q);
     auto kp = static_cast<const unsigned short*>(k);
@@ -1383,12 +1035,6 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
     auto dkp = static_cast<unsigned short*>(dk);
     auto dvp = static_cast<unsigned short*>(dv);
     const int T = g.seq_len;
-    if constexpr (D == 128) {
-        if (ds_scratch && !dq_columns.base && !dk_columns.base && !dv_columns.base)
-            return run_bwd_stored<E, D>(qp, kp, vp, op, lse, lm, gp, dqp, dkp, dvp, delta, g,
-                                        static_cast<unsigned short*>(ds_scratch), stream);
-    }
-
     hipError_t err;
     // dQ first: it also leaves D = rowsum(dO o O) in `delta` for the dK/dV kernel
     {
@@ -1457,46 +1103,35 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
                                                : plan_persistent_grid(total, k_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp,
-                               dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal, static_cast<unsigned short*>(nullptr),
-                               dk_columns, dv_columns);
+                               dvp, lm, g, k_tiles, total, tiles_per_xcd, plan.deal, dk_columns, dv_columns);
             return hipGetLastError();
         };
         const bool columns = dk_columns.base && dv_columns.base;
         if (columns != (dk_columns.base || dv_columns.base)) return hipErrorInvalidValue;
         if (g.window > 0)
-            err = columns ? launch(dkdv_split_kernel<E, D, true, true, false, true>) : launch(dkdv_split_kernel<E, D, true, true>);
+            err = columns ? launch(dkdv_split_kernel<E, D, true, true, true>) : launch(dkdv_split_kernel<E, D, true, true>);
         else if (g.causal)
-            err = columns ? launch(dkdv_split_kernel<E, D, true, false, false, true>) : launch(dkdv_split_kernel<E, D, true, false>);
+            err = columns ? launch(dkdv_split_kernel<E, D, true, false, true>) : launch(dkdv_split_kernel<E, D, true, false>);
         else
-            err = columns ? launch(dkdv_split_kernel<E, D, false, false, false, true>) : launch(dkdv_split_kernel<E, D, false, false>);
+            err = columns ? launch(dkdv_split_kernel<E, D, false, false, true>) : launch(dkdv_split_kernel<E, D, false, false>);
     }
     return err;
 }
 
 }  // namespace
 
-size_t bwd_stored_scratch_bytes(const AttnGeom& g) {
-    if (g.head_dim != 128 || g.window > 0 || !g.causal) return 0;
-    const DsBlocks blocks = DsBlocks::of(g.seq_len, g.causal != 0);
-    const long long head_bytes = blocks.per_head * DsBlocks::kElems * 2;
-    if (head_bytes > 0x7fffffffLL) return 0;  // one head's blocks are addressed through a 32-bit buffer range
-    return (size_t)head_bytes * g.packs * g.q_heads;
-}
-
 hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* v, const void* out, const float* lse,
                            RowMap lm, const void* d_out, void* dq, void* dk, void* dv, float* delta, AttnGeom g,
-                           hipStream_t stream, void* ds_scratch, ColumnSink dq_columns, ColumnSink dk_columns,
-                           ColumnSink dv_columns) {
-    if (ds_scratch && bwd_stored_scratch_bytes(g) == 0) ds_scratch = nullptr;
+                           hipStream_t stream, ColumnSink dq_columns, ColumnSink dk_columns, ColumnSink dv_columns) {
     if (type == Elem::BF16) {
-        if (g.head_dim == 64) return run_bwd<Bf16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream, dq_columns, dk_columns,
+        if (g.head_dim == 64) return run_bwd<Bf16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, stream, dq_columns, dk_columns,
                                                               dv_columns);
-        if (g.head_dim == 128) return run_bwd<Bf16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream, dq_columns, dk_columns,
+        if (g.head_dim == 128) return run_bwd<Bf16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, stream, dq_columns, dk_columns,
                                                               dv_columns);
     } else if (type == Elem::F16) {
-        if (g.head_dim == 64) return run_bwd<Fp16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream, dq_columns, dk_columns,
+        if (g.head_dim == 64) return run_bwd<Fp16, 64>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, stream, dq_columns, dk_columns,
                                                               dv_columns);
-        if (g.head_dim == 128) return run_bwd<Fp16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, ds_scratch, stream, dq_columns, dk_columns,
+        if (g.head_dim == 128) return run_bwd<Fp16, 128>(q, k, v, out, lse, lm, d_out, dq, dk, dv, delta, g, stream, dq_columns, dk_columns,
                                                               dv_columns);
     }
     return hipErrorInvalidValue;

@@ -25,7 +25,7 @@ OK, INVALID_ARGUMENT, UNSUPPORTED, RUNTIME = 0, 1, 2, 3
 F32, BF16, F16 = 0, 1, 2
 COMPUTE_AUTO = -1
 LAYOUT_COLUMNS, LAYOUT_BHTD = 0, 1
-WORKSPACE_KEEP, WORKSPACE_REUSE, BACKWARD_STORED_SCORES = 0x100, 0x200, 0x400  # OR-ed into the layout argument
+WORKSPACE_KEEP, WORKSPACE_REUSE = 0x100, 0x200  # OR-ed into the layout argument
 
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 _COMPUTE_CODE = {None: COMPUTE_AUTO, "auto": COMPUTE_AUTO, "fp32": F32, "bf16": BF16, "fp16": F16,
@@ -314,11 +314,8 @@ class HipFlashAttention:
                             value_gradient, delta_workspace, head_count, head_dimension, scale, causal=True,
                             column_start=0, column_count=0, pack_count=1, *, kv_head_count=None, compute=None,
                             workspace=None, stream=None, rope=None, window_size=0, global_token_count=0,
-                            reuse_forward_workspace=False, stored_scores=False):
+                            reuse_forward_workspace=False):
         """CudaFlashAttention::backwardMultiHead. Returns (dQ, dK, dV, delta).
-
-        stored_scores: the one-pass backward variant (SENTINEL_HIP_BACKWARD_STORED_SCORES); the workspace grows by the
-        16-bit score gradients.
 
         reuse_forward_workspace: `workspace` is the tensor a forward_multi_head(..., keep_for_backward=True) call with
         the same tensors and arguments filled; query / key / value / out are then not converted again.
@@ -344,15 +341,14 @@ class HipFlashAttention:
         value_gradient = _ensure_size(value_gradient, value.shape[0], cols, query)
         delta_workspace = _ensure_size(delta_workspace, head_count, packs * max(seq, 1), query)
         comp = _COMPUTE_CODE[compute]
-        variant = BACKWARD_STORED_SCORES if stored_scores else 0
-        ws, ws_bytes, ws_own = _workspace(lib, F32, comp, LAYOUT_COLUMNS | variant, head_count, kv_heads, head_dimension,
+        ws, ws_bytes, ws_own = _workspace(lib, F32, comp, LAYOUT_COLUMNS, head_count, kv_heads, head_dimension,
                                           max(seq, 1), packs, True, query.device, workspace)
         if reuse_forward_workspace and ws_own is not None:
             raise ValueError("HipFlashAttention::backwardMultiHead reuse_forward_workspace needs the forward call's workspace")
         _on_stream(stream, ws_own)
         head = (_ptr(query), _ptr(key), _ptr(value), _ptr(out), _ptr(log_sum_exp), _ptr(out_gradient), _ptr(query_gradient),
                 _ptr(key_gradient), _ptr(value_gradient), _ptr(delta_workspace))
-        tail = (F32, comp, LAYOUT_COLUMNS | variant | (WORKSPACE_REUSE if reuse_forward_workspace else 0), head_count, kv_heads,
+        tail = (F32, comp, LAYOUT_COLUMNS | (WORKSPACE_REUSE if reuse_forward_workspace else 0), head_count, kv_heads,
                 head_dimension, cols, column_start, column_count,
                 pack_count, float(scale), int(bool(causal)), _ptr(ws), ws_bytes, _stream_handle(stream))
         if window_size > 0 or global_token_count != 0:
@@ -469,11 +465,8 @@ def flash_attention_forward(q, k, v, scale=None, causal=True, out=None, lse=None
 
 
 def flash_attention_backward(q, k, v, out, lse, d_out, scale=None, causal=True, dq=None, dk=None, dv=None, delta=None,
-                             stream=None, window_size=0, global_token_count=0, stored_scores=False, workspace=None):
-    """Native backward on [B,H,T,d] tensors. Returns (dq, dk, dv).
-
-    stored_scores: the one-pass variant (SENTINEL_HIP_BACKWARD_STORED_SCORES): dS goes through `workspace` (allocated
-    here when not given: B * Hq * T^2 bytes under the causal mask) instead of being recomputed for dQ."""
+                             stream=None, window_size=0, global_token_count=0):
+    """Native backward on [B,H,T,d] tensors. Returns (dq, dk, dv)."""
     lib = load_library()
     b, hq, hkv, t, d = _bhtd_geometry(q, k, v)
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
@@ -492,11 +485,7 @@ def flash_attention_backward(q, k, v, out, lse, d_out, scale=None, causal=True, 
         _on_stream(stream, delta)
     code = _DTYPE_CODE[q.dtype]
     head = (_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(d_out), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(delta))
-    layout = LAYOUT_BHTD | (BACKWARD_STORED_SCORES if stored_scores else 0)
-    ws, ws_bytes, ws_own = _workspace(lib, code, COMPUTE_AUTO, layout, hq, hkv, d, t, b, True, q.device, workspace)
-    _on_stream(stream, ws_own)
-    tail = (code, COMPUTE_AUTO, layout, hq, hkv, d, 0, 0, t, b, scale, int(bool(causal)), _ptr(ws), ws_bytes,
-            _stream_handle(stream))
+    tail = (code, COMPUTE_AUTO, LAYOUT_BHTD, hq, hkv, d, 0, 0, t, b, scale, int(bool(causal)), None, 0, _stream_handle(stream))
     if window_size > 0 or global_token_count != 0:
         _check(lib.sentinel_hip_flash_bwd_sparse(*head, None, None, 0, 0, int(window_size), int(global_token_count), *tail))
     else:

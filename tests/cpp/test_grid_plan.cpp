@@ -1,6 +1,6 @@
-// Host-side check of the persistent grids' tile assignment (sentinel_amd/csrc/mfma_tile.h: tile_of_slot,
-// plan_persistent_grid).  Needs no GPU: it only runs the host copies of the index arithmetic the kernels use.
-#include "../../sentinel_amd/csrc/mfma_tile.h"
+// Host-side check of the persistent grids' tile assignment (sentinel_amd/csrc/grid_plan.h: tile_of_slot,
+// plan_persistent_grid).  Plain C++, needs neither a GPU nor the HIP compiler: it runs the index arithmetic the kernels use.
+#include "../../sentinel_amd/csrc/grid_plan.h"
 
 #include <cstdio>
 #include <vector>

@@ -121,6 +121,37 @@ int main() {
             expectInvalid("rope table too short", [&] { HipOps::rotaryRotateInPlace(x, heads, d, d / 2, ct, stb, 11); });
             expectInvalid("rope dims", [&] { HipOps::rotaryRotateInPlace(x, heads, d, 0, ct, stb); });
         }
+        // kept operands belong to the matrices they were made from: a backward call that is handed another key matrix
+        // (or another mask) together with the forward call's KeptOperands converts everything again
+        {
+            const int heads = 2, d = 64, T = 96;
+            const float scale = 0.125f;
+            unsigned st = 99u;
+            HipMatrix q, k, k2, v, g, out, lse, dq, dk, dv, delta, dq2, dk2, dv2, delta2;
+            q.upload(lcg(static_cast<size_t>(heads) * d * T, st), static_cast<size_t>(heads) * d, T);
+            k.upload(lcg(static_cast<size_t>(heads) * d * T, st), static_cast<size_t>(heads) * d, T);
+            k2.upload(lcg(static_cast<size_t>(heads) * d * T, st), static_cast<size_t>(heads) * d, T);
+            v.upload(lcg(static_cast<size_t>(heads) * d * T, st), static_cast<size_t>(heads) * d, T);
+            g.upload(lcg(static_cast<size_t>(heads) * d * T, st), static_cast<size_t>(heads) * d, T);
+            HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_BF16;
+            HipFlashAttention::KeptOperands kept;
+            HipFlashAttention::forwardMultiHead(q, k, v, out, lse, heads, d, scale, true, 0, T, 1, 0, &kept);
+            if (!kept.filled) throw std::runtime_error("forward did not keep its operands");
+            HipFlashAttention::backwardMultiHead(q, k2, v, out, lse, g, dq, dk, dv, delta, heads, d, scale, true, 0, T, 1, 0, &kept);
+            HipFlashAttention::backwardMultiHead(q, k2, v, out, lse, g, dq2, dk2, dv2, delta2, heads, d, scale, true, 0, T, 1, 0, nullptr);
+            if (dq.download() != dq2.download() || dk.download() != dk2.download() || dv.download() != dv2.download())
+                throw std::runtime_error("backward reused 16-bit copies of another key matrix");
+            HipFlashAttention::backwardMultiHead(q, k, v, out, lse, g, dq, dk, dv, delta, heads, d, scale, false, 0, T, 1, 0, &kept);
+            HipFlashAttention::backwardMultiHead(q, k, v, out, lse, g, dq2, dk2, dv2, delta2, heads, d, scale, false, 0, T, 1, 0, nullptr);
+            if (dq.download() != dq2.download() || dk.download() != dk2.download() || dv.download() != dv2.download())
+                throw std::runtime_error("backward under another mask differs with kept operands");
+            kept.invalidate();
+            HipFlashAttention::backwardMultiHead(q, k, v, out, lse, g, dq, dk, dv, delta, heads, d, scale, true, 0, T, 1, 0, &kept);
+            HipFlashAttention::backwardMultiHead(q, k, v, out, lse, g, dq2, dk2, dv2, delta2, heads, d, scale, true, 0, T, 1, 0, nullptr);
+            if (dq.download() != dq2.download()) throw std::runtime_error("backward after invalidate() differs");
+            HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
+            std::printf("  %-34s  ok\n", "kept operands tied to their tensors");
+        }
         // single-head wrappers
         HipMatrix one, o1, l1, d1, d2, d3;
         one.ensureSize(16, 40);

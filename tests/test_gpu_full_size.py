@@ -48,11 +48,11 @@ def _inputs(name):
     return q, k, v, g
 
 
-def _run(q, k, v, g, **backward_options):
+def _run(q, k, v, g):
     from sentinel_amd import flash_attention_backward, flash_attention_forward
     out, lse = flash_attention_forward(q, k, v)
     dq, dk, dv = (torch.full_like(x, float("nan")) for x in (q, k, v))
-    flash_attention_backward(q, k, v, out, lse, g, dq=dq, dk=dk, dv=dv, **backward_options)
+    flash_attention_backward(q, k, v, out, lse, g, dq=dq, dk=dk, dv=dv)
     torch.cuda.synchronize()
     return out, lse, dq, dk, dv
 
@@ -75,12 +75,13 @@ def _check_slice(name, where, out, lse, dq, dk, dv, q, k, v, g):
     hs = slice(kvh * group, (kvh + 1) * group)
     want = gpu_util.oracle(_columns(q[bi, hs]), _columns(k[bi, kvh:kvh + 1]), _columns(v[bi, kvh:kvh + 1]),
                            _columns(g[bi, hs]), group, 1, d, t, 1)
-    gpu_util.assert_close_lowp(_columns(out[bi, hs]), want["out"], "out", d)
+    tag = f"full-size {name} {where}"
+    gpu_util.assert_close_lowp(_columns(out[bi, hs]), want["out"], tag + " out", d)
     got_lse = lse[bi, hs].float().cpu().numpy()
     assert np.max(np.abs(got_lse - want["lse"][:, :t])) <= 2e-3, "lse"
-    gpu_util.assert_close_lowp(_columns(dq[bi, hs]), want["dq"], "dq", d)
-    gpu_util.assert_close_lowp(_columns(dk[bi, kvh:kvh + 1]), want["dk"], "dk", d)
-    gpu_util.assert_close_lowp(_columns(dv[bi, kvh:kvh + 1]), want["dv"], "dv", d)
+    gpu_util.assert_close_lowp(_columns(dq[bi, hs]), want["dq"], tag + " dq", d)
+    gpu_util.assert_close_lowp(_columns(dk[bi, kvh:kvh + 1]), want["dk"], tag + " dk", d)
+    gpu_util.assert_close_lowp(_columns(dv[bi, kvh:kvh + 1]), want["dv"], tag + " dv", d)
 
 
 @pytest.mark.parametrize("where", ["first", "middle", "last"])
@@ -91,19 +92,6 @@ def test_slice_matches_oracle_at_full_length(name, where):
     out, lse, dq, dk, dv = _run(q, k, v, g)
     _check_slice(name, where, out, lse, dq, dk, dv, q, k, v, g)
     for x in (out, lse, dq, dk, dv):
-        assert torch.isfinite(x.float()).all(), "non-finite value outside the checked slice"
-
-
-@pytest.mark.parametrize("where", ["first", "last"])
-@pytest.mark.parametrize("name", ["c4_gqa", "target_shape"])
-def test_stored_scores_backward_at_full_length(name, where):
-    """The one-pass backward variant (dS written by the dK / dV kernel, dQ formed from it; 2 GiB of scores at these shapes)
-    at the full size: the two ends of the grids' walk against the oracle."""
-    print(f"case {name} {where} stored-scores backward vs oracle", flush=True)
-    q, k, v, g = _inputs(name)
-    out, lse, dq, dk, dv = _run(q, k, v, g, stored_scores=True)
-    _check_slice(name, where, out, lse, dq, dk, dv, q, k, v, g)
-    for x in (dq, dk, dv):
         assert torch.isfinite(x.float()).all(), "non-finite value outside the checked slice"
 
 
