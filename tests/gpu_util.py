@@ -57,7 +57,7 @@ CASE_MARGINS = []  # (name, worst row error / max|row|, row_floor coefficient ne
 
 # D = rowsum(dO o O) enters dQ and dK only (dS = P o (dP - D)); O and dV never see it.  1.25 x the largest
 # coefficient any row of any committed case needs (conftest.py prints it per run).
-DELTA_ROW_FLOOR = 1.5e-2
+DELTA_ROW_FLOOR = 1.0e-2
 
 
 def tensor_kind(name):
