@@ -621,7 +621,7 @@ private:
     bool fusedRotation() const {
         const int compute = HipFlashAttention::computeType();
         return (compute == SENTINEL_HIP_COMPUTE_BF16 || compute == SENTINEL_HIP_COMPUTE_F16) &&
-               (headDimension == 64 || headDimension == 128);
+               headDimension % 8 == 0 && headDimension <= 128;
     }
 };
 

@@ -125,7 +125,7 @@ public:
     static constexpr int maxHeadDimension = 128;
 
     /// arithmetic for the matrix products: SENTINEL_HIP_COMPUTE_AUTO (exact fp32 for these fp32 matrices),
-    /// SENTINEL_HIP_COMPUTE_BF16 or SENTINEL_HIP_COMPUTE_F16 (MFMA, head_dim 64 / 128)
+    /// SENTINEL_HIP_COMPUTE_BF16 or SENTINEL_HIP_COMPUTE_F16 (MFMA; head_dim a multiple of 8, padded to 64 / 128 inside)
     static int& computeType() {
         static int value = SENTINEL_HIP_COMPUTE_AUTO;
         return value;

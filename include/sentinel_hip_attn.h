@@ -53,8 +53,12 @@ enum { SENTINEL_HIP_F32 = 0, SENTINEL_HIP_BF16 = 1, SENTINEL_HIP_F16 = 2 };
 enum {
     SENTINEL_HIP_COMPUTE_AUTO = -1, /* F32 io -> F32 arithmetic; BF16 / F16 io -> MFMA in that type */
     SENTINEL_HIP_COMPUTE_F32 = 0,   /* exact fp32 FMA path (any head_dim <= 128) */
-    SENTINEL_HIP_COMPUTE_BF16 = 1,  /* bf16 MFMA, fp32 accumulation (head_dim 64 or 128) */
-    SENTINEL_HIP_COMPUTE_F16 = 2    /* fp16 MFMA, fp32 accumulation (head_dim 64 or 128) */
+    SENTINEL_HIP_COMPUTE_BF16 = 1,  /* bf16 MFMA, fp32 accumulation: the kernels are tiled for head_dim 64 and 128; fp32
+                                       column tensors of any head_dim that is a multiple of 8 (<= 128) run on them too,
+                                       zero-padded to 64 / 128 by the conversion pass they go through anyway (the CUDA
+                                       path's generic kernel takes any head_dim <= 64, CudaFlashAttention.cu:1596-1599);
+                                       16-bit [B,H,T,d] tensors need head_dim 64 or 128 */
+    SENTINEL_HIP_COMPUTE_F16 = 2    /* fp16 MFMA, fp32 accumulation: same rules */
 };
 
 /*

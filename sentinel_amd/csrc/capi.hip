@@ -39,6 +39,7 @@ struct Resolved {
     long long stride;  // column layout only
     int column_start;
     bool adapter;  // column layout fp32 tensors converted to [B,H,T,d] 16-bit for the MFMA kernels
+    int source_dim;  // the caller's head dim; g.head_dim is larger when the conversion pads it to a tiling the MFMA kernels have
     bool keep;     // forward: lay the converted operands out where the backward expects them (SENTINEL_HIP_WORKSPACE_KEEP)
     bool reuse;    // backward: q, k, v, out of the workspace are the forward's (SENTINEL_HIP_WORKSPACE_REUSE)
 };
@@ -83,13 +84,16 @@ int resolve(const char* op, int io_dtype, int compute_dtype, int layout, int q_h
         if (io_dtype != SENTINEL_HIP_F32)
             return fail(SENTINEL_HIP_UNSUPPORTED, "%s fp32 arithmetic needs fp32 tensors", op);
     } else {
-        if (!mfma_supported(head_dim))
-            return fail(SENTINEL_HIP_UNSUPPORTED, "%s MFMA kernels cover head_dim 64 and 128, got %d", op, head_dim);
         if (io_dtype == SENTINEL_HIP_F32) {
             if (layout != SENTINEL_HIP_LAYOUT_COLUMNS)
                 return fail(SENTINEL_HIP_UNSUPPORTED, "%s fp32 tensors with MFMA arithmetic need the column layout", op);
+            // the conversion pass pads head dims without a tiling of their own with zeros (no product changes)
+            if (mfma_padded_head_dim(head_dim) == 0)
+                return fail(SENTINEL_HIP_UNSUPPORTED, "%s MFMA arithmetic needs a head_dim that is a multiple of 8, got %d", op, head_dim);
             adapter = true;
         } else {
+            if (!mfma_supported(head_dim))
+                return fail(SENTINEL_HIP_UNSUPPORTED, "%s 16-bit tensors: the MFMA kernels cover head_dim 64 and 128, got %d", op, head_dim);
             if (io_dtype != compute)
                 return fail(SENTINEL_HIP_UNSUPPORTED, "%s 16-bit tensors must be multiplied in their own type", op);
             if (layout != SENTINEL_HIP_LAYOUT_BHTD)
@@ -101,13 +105,15 @@ int resolve(const char* op, int io_dtype, int compute_dtype, int layout, int q_h
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s too many columns", op);
     if (compute != SENTINEL_HIP_COMPUTE_F32) {
         // the MFMA kernels address one head through a 32-bit buffer range and int byte offsets inside it
-        if ((long long)seq_len * head_dim * 2 > 0x7fffffffLL)
+        if ((long long)seq_len * (adapter ? mfma_padded_head_dim(head_dim) : head_dim) * 2 > 0x7fffffffLL)
             return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s one head exceeds 2 GiB (seq_len * head_dim * 2 bytes)", op);
         // the layout conversion launches one grid plane per (pack, head)
         if (adapter && (long long)pack_count * q_heads > 65535)
             return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s more than 65535 (pack, head) pairs in the column layout", op);
     }
 
+    r->source_dim = head_dim;
+    if (adapter) head_dim = mfma_padded_head_dim(head_dim);
     r->g = AttnGeom{q_heads, kv_heads, head_dim, seq_len, pack_count, scale, causal ? 1 : 0, 0, 0};
     r->io = io_dtype;
     r->compute = compute;
@@ -229,7 +235,7 @@ const RopeRequest kNoRope = {nullptr, nullptr, 0, 0, false};
 int resolve_rope(const char* op, const RopeRequest& req, const Resolved& r, RopeTables* rope) {
     *rope = RopeTables{nullptr, nullptr, 0, 0};
     if (!req.requested) return SENTINEL_HIP_OK;
-    const int rc = check_rope(op, req.cos, req.sin, req.table_positions, r.g.head_dim, req.position_offset, r.g.seq_len);
+    const int rc = check_rope(op, req.cos, req.sin, req.table_positions, r.source_dim, req.position_offset, r.g.seq_len);
     if (rc != SENTINEL_HIP_OK) return rc;
     if (misaligned(req.cos) || misaligned(req.sin))
         return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s rope tables must be 16-byte aligned", op);
@@ -314,16 +320,16 @@ int flash_fwd(const char* op, const void* q, const void* k, const void* v, void*
     in.job[0] = ConvertJob{static_cast<const float*>(q) + off, static_cast<unsigned short*>(q16), g.q_heads, 1, 0};
     in.job[1] = ConvertJob{static_cast<const float*>(k) + off, static_cast<unsigned short*>(k16), g.kv_heads, 1, 0};
     in.job[2] = ConvertJob{static_cast<const float*>(v) + off, static_cast<unsigned short*>(v16), g.kv_heads, 0, 0};
-    hipError_t err = launch_columns_to_bhtd_jobs(type, in, g.head_dim, stride, g.seq_len, g.packs, rope, stream);
+    hipError_t err = launch_columns_to_bhtd_jobs(type, in, r.source_dim, stride, g.seq_len, g.packs, rope, stream, g.head_dim);
     // O goes to the caller's matrix straight from the kernel's accumulators (and in 16 bit to the workspace, for the
     // backward); a conversion pass only where the kernel's 32-bit row offsets would not reach
     const bool direct = direct_columns(r);
     if (err == hipSuccess)
         err = launch_fwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g, stream,
-                              direct ? ColumnSink{static_cast<float*>(out) + off, r.stride, none} : kNoColumnSink);
+                              direct ? ColumnSink{static_cast<float*>(out) + off, r.stride, none, r.source_dim} : kNoColumnSink);
     if (err == hipSuccess && !direct)
-        err = launch_bhtd_to_columns(type, o16, static_cast<float*>(out) + off, g.q_heads, g.head_dim, stride, g.seq_len,
-                                     g.packs, none, stream);
+        err = launch_bhtd_to_columns(type, o16, static_cast<float*>(out) + off, g.q_heads, r.source_dim, stride, g.seq_len,
+                                     g.packs, none, stream, g.head_dim);
     if (err != hipSuccess) return fail_hip("MFMA forward (column layout) launch", err);
     return SENTINEL_HIP_OK;
 }
@@ -400,30 +406,30 @@ int flash_bwd(const char* op, const void* q, const void* k, const void* v, const
         in.job[in.count++] = ConvertJob{static_cast<const float*>(k) + off, static_cast<unsigned short*>(k16), g.kv_heads, 1, 0};
         in.job[in.count++] = ConvertJob{static_cast<const float*>(v) + off, static_cast<unsigned short*>(v16), g.kv_heads, 0, 0};
     }
-    hipError_t err = launch_columns_to_bhtd_jobs(type, in, g.head_dim, stride, T, g.packs, rope, stream);
+    hipError_t err = launch_columns_to_bhtd_jobs(type, in, r.source_dim, stride, T, g.packs, rope, stream, g.head_dim);
     // The gradients leave the kernels as fp32 columns, straight from the accumulators, rotated back on the way (they are
     // gradients with respect to the unrotated Q, K).  Matrices beyond the kernels' 32-bit row offsets write 16-bit
     // tensors and convert them in passes of their own.
     if (direct_columns(r)) {
         if (err == hipSuccess)
             err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream,
-                                  ColumnSink{static_cast<float*>(dq) + off, r.stride, rope},
-                                  ColumnSink{static_cast<float*>(dk) + off, r.stride, rope},
-                                  ColumnSink{static_cast<float*>(dv) + off, r.stride, none});
+                                  ColumnSink{static_cast<float*>(dq) + off, r.stride, rope, r.source_dim},
+                                  ColumnSink{static_cast<float*>(dk) + off, r.stride, rope, r.source_dim},
+                                  ColumnSink{static_cast<float*>(dv) + off, r.stride, none, r.source_dim});
         if (err != hipSuccess) return fail_hip("MFMA backward (column layout) launch", err);
         return SENTINEL_HIP_OK;
     }
     if (err == hipSuccess)
         err = launch_bwd_mfma(type, q16, k16, v16, o16, lse + off, lse_map(r), g16, dq16, dk16, dv16, delta, g, stream);
     if (err == hipSuccess)
-        err = launch_bhtd_to_columns(type, dq16, static_cast<float*>(dq) + off, g.q_heads, g.head_dim, stride, T, g.packs,
-                                     rope, stream);
+        err = launch_bhtd_to_columns(type, dq16, static_cast<float*>(dq) + off, g.q_heads, r.source_dim, stride, T, g.packs,
+                                     rope, stream, g.head_dim);
     if (err == hipSuccess)
-        err = launch_bhtd_to_columns(type, dk16, static_cast<float*>(dk) + off, g.kv_heads, g.head_dim, stride, T, g.packs,
-                                     rope, stream);
+        err = launch_bhtd_to_columns(type, dk16, static_cast<float*>(dk) + off, g.kv_heads, r.source_dim, stride, T, g.packs,
+                                     rope, stream, g.head_dim);
     if (err == hipSuccess)
-        err = launch_bhtd_to_columns(type, dv16, static_cast<float*>(dv) + off, g.kv_heads, g.head_dim, stride, T, g.packs,
-                                     none, stream);
+        err = launch_bhtd_to_columns(type, dv16, static_cast<float*>(dv) + off, g.kv_heads, r.source_dim, stride, T, g.packs,
+                                     none, stream, g.head_dim);
     if (err != hipSuccess) return fail_hip("MFMA backward (column layout) launch", err);
     return SENTINEL_HIP_OK;
 }

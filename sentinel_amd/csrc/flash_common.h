@@ -70,15 +70,23 @@ struct RopeTables {
 // consecutive tokens per register, which is 128 contiguous bytes of a row of that matrix: no conversion pass is
 // needed on the way out.  `base` is already advanced to the first column of pack 0; pack p starts seq_len columns on.
 // `inverse_rope`: the rotary embedding's inverse applied on the way (dQ, dK), as bhtd_to_columns does.
+// `head_dim`: rows per head of that matrix (a multiple of 8); where it is smaller than the kernels' own head dim (operands
+// zero-padded to the next tiling, see launch_columns_to_bhtd_jobs) only that many head dims are written.
 struct ColumnSink {
     float* base;
     long long stride;  // columns per row
     RopeTables inverse_rope;
+    int head_dim;
 };
-constexpr ColumnSink kNoColumnSink = {nullptr, 0, {nullptr, nullptr, 0, 0}};
+constexpr ColumnSink kNoColumnSink = {nullptr, 0, {nullptr, nullptr, 0, 0}, 0};
 
 // ---- MFMA path (flash_mfma_*.hip): bf16 / fp16 [B,H,T,d] tensors, head_dim 64 or 128 ----
 bool mfma_supported(int head_dim);
+// the tiling a head dim is zero-padded to when it has none of its own (multiples of 8 up to 128), 0 if there is none
+inline int mfma_padded_head_dim(int head_dim) {
+    if (head_dim <= 0 || head_dim > 128 || head_dim % 8 != 0) return 0;
+    return head_dim <= 64 ? 64 : 128;
+}
 // lse rows are addressed through `lm`; delta is q_heads x (packs * seq_len).
 // out_columns: O is written there as well (the 16-bit `out` is always written: the backward reads it)
 hipError_t launch_fwd_mfma(Elem type, const void* q, const void* k, const void* v, void* out, float* lse, RowMap lm,
@@ -92,7 +100,8 @@ hipError_t launch_bwd_mfma(Elem type, const void* q, const void* k, const void* 
 
 // ---- layout adapter (layout_adapter.hip): Sentinel column layout fp32 <-> [B,H,T,d] bf16 / fp16 ----
 // several tensors of one shape family (same head_dim, stride, sequence length, packs; head counts may differ) through one
-// launch; `rotate`: apply the rotary tables to this tensor; z_end is filled in by the launcher
+// launch; `rotate`: apply the rotary tables to this tensor; z_end is filled in by the launcher.  padded_dim (0: head_dim):
+// head dims per token on the 16-bit side, the ones from head_dim on are zeros (written / skipped)
 constexpr int kMaxConvertJobs = 5;
 struct ConvertJob {
     const float* src;     // first column of pack 0
@@ -106,11 +115,11 @@ struct ConvertJobs {
     int count;
 };
 hipError_t launch_columns_to_bhtd_jobs(Elem type, ConvertJobs jobs, int head_dim, int stride_columns, int seq_len, int packs,
-                                       RopeTables rope, hipStream_t stream);
+                                       RopeTables rope, hipStream_t stream, int padded_dim = 0);
 hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int heads, int head_dim, int stride_columns,
-                                  int seq_len, int packs, RopeTables rope, hipStream_t stream);
+                                  int seq_len, int packs, RopeTables rope, hipStream_t stream, int padded_dim = 0);
 hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,
-                                  int seq_len, int packs, RopeTables inverse_rope, hipStream_t stream);
+                                  int seq_len, int packs, RopeTables inverse_rope, hipStream_t stream, int padded_dim = 0);
 // single-query attention against the K/V cache (fp32 column layout, `stride` positions per row, `length` used)
 size_t decode_workspace_bytes(int q_heads, int head_dim, int length);
 // window / global_tokens: the layer's sparse mask for the query at position length - 1 (window <= 0: none)

@@ -40,13 +40,14 @@ constexpr int kSchedDsRead = 0x100;
 template <int D>
 __device__ __forceinline__ void store_block_to_sink(const f32x16 (&acc)[D / 32], float factor, const ColumnSink& sink, int head,
                                                     int pack, int token0, int seq_len, int lane) {
-    float* head_rows = sink.base + (long long)head * D * sink.stride + (long long)pack * seq_len + token0;
+    float* head_rows = sink.base + (long long)head * sink.head_dim * sink.stride + (long long)pack * seq_len + token0;
     if (sink.inverse_rope.cos)
-        store_columns_f32<D, true>(acc, factor, head_rows, (int)sink.stride, seq_len - token0, lane, sink.inverse_rope.cos,
-                                   sink.inverse_rope.sin, sink.inverse_rope.offset + token0,
+        store_columns_f32<D, true>(acc, factor, head_rows, (int)sink.stride, seq_len - token0, sink.head_dim, lane,
+                                   sink.inverse_rope.cos, sink.inverse_rope.sin, sink.inverse_rope.offset + token0,
                                    sink.inverse_rope.positions - (sink.inverse_rope.offset + token0));
     else
-        store_columns_f32<D, false>(acc, factor, head_rows, (int)sink.stride, seq_len - token0, lane, nullptr, nullptr, 0, 0);
+        store_columns_f32<D, false>(acc, factor, head_rows, (int)sink.stride, seq_len - token0, sink.head_dim, lane, nullptr,
+                                    nullptr, 0, 0);
 }
 constexpr int kOperandLead = 4;
 

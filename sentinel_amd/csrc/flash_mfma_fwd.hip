@@ -292,8 +292,9 @@ __global__ __launch_bounds__(kFwdThreads, D <= 64 ? 3 : 2) void fwd_mfma_kernel(
                              out + ((long long)b * g.q_heads + h) * T * D + (long long)q0w * D, T - q0w, lane);
     // the caller's fp32 column matrix, if it keeps O that way: straight from the accumulators, unrounded
     if (out_columns.base)
-        store_columns_f32<D, false>(acc, inv, out_columns.base + (long long)h * D * out_columns.stride + (long long)b * T + q0w,
-                                    (int)out_columns.stride, T - q0w, lane, nullptr, nullptr, 0, 0);
+        store_columns_f32<D, false>(acc, inv,
+                                    out_columns.base + (long long)h * out_columns.head_dim * out_columns.stride + (long long)b * T + q0w,
+                                    (int)out_columns.stride, T - q0w, out_columns.head_dim, lane, nullptr, nullptr, 0, 0);
     if (qrow < T && gh == 0)
         lse[b * lm.pack_stride + h * lm.head_stride + qrow] = m_run * g.scale + (l_tot > 0.0f ? __logf(l_tot) : 0.0f);
     }  // next tile of this workgroup (the last trip ended with a barrier: the LDS stages are free)

@@ -40,11 +40,14 @@ __device__ __forceinline__ void rotate_pair(float& even, float& odd, float c, fl
 // token-major side (fp32, 4 tokens per thread) and the dim-major side (16 bit, 8 dims = 16 bytes per thread)
 // both touch 64 different banks per wavefront access.  VEC4: the fp32 rows can be accessed as aligned float4
 // (pointer, stride and sequence length all multiples of 4 floats); otherwise the same code runs on scalars.
+// The 16-bit side may be wider than the fp32 side (d_out > d, both multiples of 8): head dims the MFMA kernels have no
+// tiling for are padded with zeros to the next one they have, which changes no product.
 // Up to kMaxConvertJobs tensors of one call (Q, K, V; or Q, O, K, V, dO) go through one launch: at the sequence lengths
 // Sentinel trains with a conversion takes about as long as its launch, and three to five of them were 40 % of a step.
 // grid.z runs over the (pack, head) pairs of all jobs one after the other; z_end is the running total.
 template <typename E, bool VEC4>
-__global__ __launch_bounds__(256) void columns_to_bhtd_kernel(ConvertJobs jobs, int d, long long stride, int T, RopeTables tables) {
+__global__ __launch_bounds__(256) void columns_to_bhtd_kernel(ConvertJobs jobs, int d, int d_out, long long stride, int T,
+                                                               RopeTables tables) {
     __shared__ float tile[kTile][kTile + 1];
     const int t0 = blockIdx.x * kTile;
     const int c0 = blockIdx.y * kTile;
@@ -87,11 +90,11 @@ __global__ __launch_bounds__(256) void columns_to_bhtd_kernel(ConvertJobs jobs, 
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int t = i * 32 + tid / 8;
-        if (t0 + t < T && c0 + c8 < d) {
+        if (t0 + t < T && c0 + c8 < d_out) {  // head dims [d, d_out) are written as zeros (the load phase left them zero)
             float x[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = tile[c8 + e][t];
-            if (rope.cos) {
+            if (rope.cos && c0 + c8 < d) {
                 const long long at = (long long)(rope.offset + t0 + t) * (d / 2) + (c0 + c8) / 2;
                 const float4 c = *reinterpret_cast<const float4*>(rope.cos + at);
                 const float4 sn = *reinterpret_cast<const float4*>(rope.sin + at);
@@ -103,14 +106,15 @@ __global__ __launch_bounds__(256) void columns_to_bhtd_kernel(ConvertJobs jobs, 
             u32x4 w;
 #pragma unroll
             for (int e = 0; e < 4; ++e) w[e] = E::pack2(x[2 * e], x[2 * e + 1]);
-            *reinterpret_cast<u32x4*>(dst + (((long long)b * heads + h) * T + t0 + t) * d + c0 + c8) = w;
+            *reinterpret_cast<u32x4*>(dst + (((long long)b * heads + h) * T + t0 + t) * d_out + c0 + c8) = w;
         }
     }
 }
 
 template <typename E, bool VEC4>
 __global__ __launch_bounds__(256) void bhtd_to_columns_kernel(const unsigned short* __restrict__ src, float* __restrict__ dst,
-                                                               int heads, int d, long long stride, int T, RopeTables rope) {
+                                                               int heads, int d, int d_in, long long stride, int T,
+                                                               RopeTables rope) {
     __shared__ float tile[kTile][kTile + 1];
     const int t0 = blockIdx.x * kTile;
     const int c0 = blockIdx.y * kTile;
@@ -122,7 +126,7 @@ __global__ __launch_bounds__(256) void bhtd_to_columns_kernel(const unsigned sho
     for (int i = 0; i < 2; ++i) {
         const int t = i * 32 + tid / 8;
         if (t0 + t < T && c0 + c8 < d) {
-            const u32x4 w = *reinterpret_cast<const u32x4*>(src + (((long long)b * heads + h) * T + t0 + t) * d + c0 + c8);
+            const u32x4 w = *reinterpret_cast<const u32x4*>(src + (((long long)b * heads + h) * T + t0 + t) * d_in + c0 + c8);
             float x[8];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -203,8 +207,10 @@ static bool rows_vec4(const void* base, int stride_columns, int seq_len) {
 }
 
 hipError_t launch_columns_to_bhtd_jobs(Elem type, ConvertJobs jobs, int head_dim, int stride_columns, int seq_len, int packs,
-                                       RopeTables rope, hipStream_t stream) {
-    if (jobs.count <= 0 || jobs.count > kMaxConvertJobs || head_dim % 8 != 0) return hipErrorInvalidValue;
+                                       RopeTables rope, hipStream_t stream, int padded_dim) {
+    if (padded_dim <= 0) padded_dim = head_dim;
+    if (jobs.count <= 0 || jobs.count > kMaxConvertJobs || head_dim % 8 != 0 || padded_dim % 8 != 0 || padded_dim < head_dim)
+        return hipErrorInvalidValue;
     bool v4 = true;
     long long z = 0;
     for (int i = 0; i < jobs.count; ++i) {
@@ -218,16 +224,17 @@ hipError_t launch_columns_to_bhtd_jobs(Elem type, ConvertJobs jobs, int head_dim
             one.count = 1;
             one.job[0] = jobs.job[i];
             if ((long long)packs * one.job[0].heads > 65535) return hipErrorInvalidValue;
-            const hipError_t err = launch_columns_to_bhtd_jobs(type, one, head_dim, stride_columns, seq_len, packs, rope, stream);
+            const hipError_t err = launch_columns_to_bhtd_jobs(type, one, head_dim, stride_columns, seq_len, packs, rope, stream,
+                                                               padded_dim);
             if (err != hipSuccess) return err;
         }
         return hipSuccess;
     }
-    const dim3 grid((seq_len + kTile - 1) / kTile, (head_dim + kTile - 1) / kTile, (unsigned)z);
+    const dim3 grid((seq_len + kTile - 1) / kTile, (padded_dim + kTile - 1) / kTile, (unsigned)z);
     KernelTimer timer("columns_to_bhtd", stream);
 #define SENTINEL_LAUNCH(E, V) \
-    hipLaunchKernelGGL((columns_to_bhtd_kernel<E, V>), grid, dim3(256), 0, stream, jobs, head_dim, (long long)stride_columns, \
-                       seq_len, rope)
+    hipLaunchKernelGGL((columns_to_bhtd_kernel<E, V>), grid, dim3(256), 0, stream, jobs, head_dim, padded_dim, \
+                       (long long)stride_columns, seq_len, rope)
     if (type == Elem::BF16) {
         if (v4) SENTINEL_LAUNCH(Bf16, true); else SENTINEL_LAUNCH(Bf16, false);
     } else if (type == Elem::F16) {
@@ -240,22 +247,23 @@ hipError_t launch_columns_to_bhtd_jobs(Elem type, ConvertJobs jobs, int head_dim
 }
 
 hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int heads, int head_dim, int stride_columns,
-                                  int seq_len, int packs, RopeTables rope, hipStream_t stream) {
+                                  int seq_len, int packs, RopeTables rope, hipStream_t stream, int padded_dim) {
     ConvertJobs jobs;
     jobs.count = 1;
     jobs.job[0] = ConvertJob{src, static_cast<unsigned short*>(dst), heads, rope.cos != nullptr, 0};
-    return launch_columns_to_bhtd_jobs(type, jobs, head_dim, stride_columns, seq_len, packs, rope, stream);
+    return launch_columns_to_bhtd_jobs(type, jobs, head_dim, stride_columns, seq_len, packs, rope, stream, padded_dim);
 }
 
 hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,
-                                  int seq_len, int packs, RopeTables rope, hipStream_t stream) {
+                                  int seq_len, int packs, RopeTables rope, hipStream_t stream, int padded_dim) {
+    if (padded_dim <= 0) padded_dim = head_dim;
     const dim3 grid((seq_len + kTile - 1) / kTile, (head_dim + kTile - 1) / kTile, packs * heads);
     auto in = static_cast<const unsigned short*>(src);
-    if (head_dim % 8 != 0) return hipErrorInvalidValue;
+    if (head_dim % 8 != 0 || padded_dim % 8 != 0 || padded_dim < head_dim) return hipErrorInvalidValue;
     const bool v4 = rows_vec4(dst, stride_columns, seq_len);
     KernelTimer timer("bhtd_to_columns", stream);
 #define SENTINEL_LAUNCH(E, V) \
-    hipLaunchKernelGGL((bhtd_to_columns_kernel<E, V>), grid, dim3(256), 0, stream, in, dst, heads, head_dim, \
+    hipLaunchKernelGGL((bhtd_to_columns_kernel<E, V>), grid, dim3(256), 0, stream, in, dst, heads, head_dim, padded_dim, \
                        (long long)stride_columns, seq_len, rope)
     if (type == Elem::BF16) {
         if (v4) SENTINEL_LAUNCH(Bf16, true); else SENTINEL_LAUNCH(Bf16, false);

@@ -311,10 +311,12 @@ __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], 
 // dim's row is a scalar offset; D * stride * 4 must stay below 2^31 (the host checks).
 // ROTATE: each (even, odd) pair of head dims is rotated back by the angle of its token's position (table row
 // `position0 + n`), in fp32 without fused multiply-adds, exactly as the conversion pass bhtd_to_columns does.
+// valid_dims: head dims the matrix has per head (a multiple of 8, <= D): the kernels' padding dims are not written, and
+// the rotary tables have valid_dims / 2 entries per position.
 template <int D, bool ROTATE>
 __device__ __forceinline__ void store_columns_f32(const f32x16 (&acc)[D / 32], float factor, float* head_rows, int stride,
-                                                  int valid_rows, int lane, const float* cos_table, const float* sin_table,
-                                                  int position0, int table_rows_left) {
+                                                  int valid_rows, int valid_dims, int lane, const float* cos_table,
+                                                  const float* sin_table, int position0, int table_rows_left) {
 #pragma clang fp contract(off)
     asm volatile("" : "+v"(lane));  // keeps the per-lane address arithmetic here instead of hoisted over the caller's loops
     const int n = lane % 32;
@@ -326,19 +328,20 @@ __device__ __forceinline__ void store_columns_f32(const f32x16 (&acc)[D / 32], f
     int table_bytes = 0;
     if (ROTATE) {
         // the tables' rows from position0 on, with their true extent
-        const long long extent = (long long)table_rows_left * (D / 2) * 4;
+        const long long extent = (long long)table_rows_left * (valid_dims / 2) * 4;
         const int records = extent > 0x7fffffffLL ? 0x7fffffff : (int)extent;
-        cos_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(cos_table) + (long long)position0 * (D / 2), 0, records,
-                                                     0x00020000);
-        sin_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sin_table) + (long long)position0 * (D / 2), 0, records,
-                                                     0x00020000);
-        table_bytes = n * (D / 2) * 4;
+        cos_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(cos_table) + (long long)position0 * (valid_dims / 2), 0,
+                                                     records, 0x00020000);
+        sin_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sin_table) + (long long)position0 * (valid_dims / 2), 0,
+                                                     records, 0x00020000);
+        table_bytes = n * (valid_dims / 2) * 4;
     }
 #pragma unroll
     for (int cb = 0; cb < D / 32; ++cb)
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const int dim = cb * 32 + a * 8;  // + gh * 4 through the lane's offset
+            if (dim >= valid_dims) continue;  // (wavefront-uniform)
             float x[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) x[j] = acc[cb][a * 4 + j] * factor;

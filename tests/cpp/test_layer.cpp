@@ -243,6 +243,9 @@ int main() {
         // MFMA arithmetic for the attention core (projections stay fp32), rotation fused into the conversion passes
         runCase("bf16 E256 H4 d64 T128 packs2", 256, 4, 4, 64, 128, 2, SENTINEL_HIP_COMPUTE_BF16, 2e-2f);
         runCase("fp16 GQA E256 4q/1kv d128 T200", 256, 4, 1, 128, 200, 1, SENTINEL_HIP_COMPUTE_F16, 2e-2f);
+        // head dims without a tiling of their own (zero-padded to 64 / 128 inside the conversion pass), rotation fused
+        runCase("bf16 E288 H3 d96 T130 packs2", 288, 3, 3, 96, 130, 2, SENTINEL_HIP_COMPUTE_BF16, 2e-2f);
+        runCase("fp16 GQA E128 4q/2kv d32 T70", 128, 4, 2, 32, 70, 1, SENTINEL_HIP_COMPUTE_F16, 2e-2f);
         // the sparse mask: the shape of runSparseComputeSmokeDemo (E=32, H=2, T=16, W=4, G=2) and larger ones
         HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
         runCase("sparse fp32 E32 H2 d16 T16 W4 G2", 32, 2, 2, 16, 16, 1, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 4, 2);

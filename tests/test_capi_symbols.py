@@ -51,7 +51,10 @@ def test_codes_and_messages_without_a_gpu(lib):
     assert call(col0=190) == 1 and b"invalid column window" in lib.sentinel_hip_last_error()
     assert call(packs=5) == 1 and b"pack window exceeds columns" in lib.sentinel_hip_last_error()
     assert call(scale=0.0) == 1 and b"scale must be positive" in lib.sentinel_hip_last_error()
-    assert call(comp=1) == 2 and b"head_dim 64 and 128" in lib.sentinel_hip_last_error()   # d=16 has no MFMA kernel
+    # MFMA arithmetic pads head dims to 64 / 128 in the conversion pass of fp32 column tensors: multiples of 8 only,
+    # and 16-bit [B,H,T,d] tensors (no conversion pass) need a head dim the kernels are tiled for
+    assert call(comp=1, d=12, stride=192) == 2 and b"multiple of 8" in lib.sentinel_hip_last_error()
+    assert call(io=1, layout=1, d=16) == 2 and b"head_dim 64 and 128" in lib.sentinel_hip_last_error()
     assert call(io=1, layout=0, d=64) == 2                                        # 16-bit needs [B,H,T,d]
     # a valid call without a device is a runtime error, not a silent fallback
     if not lib.sentinel_hip_device_available():

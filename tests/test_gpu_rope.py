@@ -40,7 +40,10 @@ def test_rope_rotate_is_bit_identical_to_the_oracle(shape, inverse):
 # off the multiples of 32, windows that start and end inside a matrix, and tables that end exactly at the last position
 @pytest.mark.parametrize("shape", [(4, 4, 64, 128, 1, 0, 0, 0, 3), (8, 2, 128, 200, 2, 4, 4, 0, 3), (2, 1, 64, 70, 3, 3, 1, 11, 3),
                                    (2, 1, 128, 33, 2, 5, 3, 2, 0), (4, 2, 64, 257, 1, 1, 0, 0, 0), (3, 3, 128, 31, 3, 0, 2, 9, 0),
-                                   (2, 2, 64, 1, 2, 2, 1, 0, 0)])
+                                   (2, 2, 64, 1, 2, 2, 1, 0, 0),
+                                   # head dims padded to the kernels' tilings: the tables keep head_dim / 2 entries per position
+                                   (4, 2, 32, 150, 2, 0, 0, 0, 3), (4, 4, 96, 130, 1, 2, 3, 5, 0), (2, 1, 80, 70, 2, 0, 1, 0, 0),
+                                   (2, 2, 16, 48, 3, 1, 0, 2, 1)])
 def test_fused_rope_attention_matches_oracle(compute, shape):
     from sentinel_amd import HipFlashAttention
     hq, hkv, d, t, packs, col0, pad, offset, spare = shape

@@ -35,7 +35,11 @@ def test_cpp_attention_layer_parity_and_exceptions():
 
 
 @pytest.mark.parametrize("compute", ["bf16", "fp16"])
-@pytest.mark.parametrize("shape", [(12, 12, 64, 128, 1, 0, 0), (8, 2, 128, 200, 2, 4, 4), (2, 2, 64, 70, 3, 3, 1)])
+# (q heads, kv heads, head_dim, T, packs, first column, columns behind the window); head dims the kernels have no tiling of
+# their own for (32, 80, 96, 16, 24, 120, 72) are zero-padded to 64 / 128 by the conversion pass
+@pytest.mark.parametrize("shape", [(12, 12, 64, 128, 1, 0, 0), (8, 2, 128, 200, 2, 4, 4), (2, 2, 64, 70, 3, 3, 1),
+                                   (4, 2, 32, 150, 2, 0, 0), (8, 8, 96, 130, 1, 2, 3), (4, 1, 80, 257, 1, 0, 0),
+                                   (3, 3, 16, 48, 4, 0, 0), (2, 2, 24, 65, 2, 1, 0), (2, 1, 120, 100, 1, 0, 5), (2, 2, 72, 33, 2, 3, 0)])
 def test_columns_layout_with_mfma_arithmetic(compute, shape):
     from sentinel_amd import HipFlashAttention
     hq, hkv, d, t, packs, col0, pad = shape
@@ -67,9 +71,9 @@ def test_columns_layout_with_mfma_arithmetic(compute, shape):
 
 def test_unsupported_head_dim_is_reported_not_faked():
     from sentinel_amd import HipFlashAttention
-    q = torch.zeros((4 * 48, 64), device="cuda")
-    with pytest.raises(ValueError, match="MFMA kernels cover head_dim 64 and 128"):
-        HipFlashAttention.forward_multi_head(q, q, q, None, None, 4, 48, 0.1, compute="bf16")
+    q = torch.zeros((4 * 44, 64), device="cuda")
+    with pytest.raises(ValueError, match="head_dim that is a multiple of 8"):
+        HipFlashAttention.forward_multi_head(q, q, q, None, None, 4, 44, 0.1, compute="bf16")
     # the exact fp32 kernels take any head_dim <= 128
     out, lse = HipFlashAttention.forward_multi_head(q + 0.01, q, q, None, None, 4, 48, 0.1)
     assert torch.isfinite(out).all()
