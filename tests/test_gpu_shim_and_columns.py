@@ -75,7 +75,7 @@ def test_unsupported_head_dim_is_reported_not_faked():
     with pytest.raises(ValueError, match="head_dim that is a multiple of 8"):
         HipFlashAttention.forward_multi_head(q, q, q, None, None, 4, 44, 0.1, compute="bf16")
     # the exact fp32 kernels take any head_dim <= 128
-    out, lse = HipFlashAttention.forward_multi_head(q + 0.01, q, q, None, None, 4, 48, 0.1)
+    out, lse = HipFlashAttention.forward_multi_head(q + 0.01, q, q, None, None, 4, 44, 0.1)
     assert torch.isfinite(out).all()
 
 
