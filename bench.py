@@ -375,6 +375,28 @@ def sparse_path(torch, name, steps):
     return report
 
 
+def library_gemm(torch, dtype, n=8192, calls=30):
+    """The vendor library's plain n^3 GEMM (torch.matmul -> hipBLASLt) in the workload's 16-bit type, timed like the
+    kernels: the matrix throughput this box sustains on a full-chip GEMM under its clock and power management, to read
+    the attention kernels' fraction of the nominal peak against."""
+    tdt = {"bf16": torch.bfloat16, "fp16": torch.float16}[dtype]
+    a = torch.randn(n, n, device="cuda").to(tdt)
+    b = torch.randn(n, n, device="cuda").to(tdt)
+    c = torch.empty(n, n, device="cuda", dtype=tdt)
+    for _ in range(5):
+        torch.matmul(a, b, out=c)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(calls):
+        torch.matmul(a, b, out=c)
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / calls
+    tf = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+    return {"shape": [n, n, n], "dtype": dtype, "ms": ms, "tflops": tf, "pct_of_mfma_peak": 100.0 * tf / PEAK_TFLOPS[dtype]}
+
+
 def profiler_attached():
     """True under rocprofv3 (its preloaded tool library has initialised the GPU before this program started, and a
     process that has done so must not start another program)."""
@@ -440,6 +462,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB -> 1 GiB elementwise copy kernel three times, so that a counter run "
                          "(FETCH_SIZE / WRITE_SIZE) of this command holds a kernel of known traffic to scale by")
+    ap.add_argument("--no-gemm-calibration", action="store_true",
+                    help="skip timing the vendor library's plain 8192^3 16-bit GEMM (\"device.library_gemm\": what the "
+                         "matrix pipes of this very box sustain under its power limit; skipped by itself under a profiler)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only; attention shards over (batch, kv-head group) with no "
@@ -484,6 +509,8 @@ def main():
             torch.mul(src, 1.0, out=dst)
         torch.cuda.synchronize()
         del src, dst
+    if not args.no_gemm_calibration and not profiler_attached() and w.dtype != "fp32":
+        device["library_gemm"] = library_gemm(torch, w.dtype)
     total_flops = 7.0 * w.unit_flops
     value = total_flops / (ms_step * 1e-3) / 1e12
     peak = PEAK_TFLOPS[w.dtype]
