@@ -407,7 +407,8 @@ def profiler_attached():
 def layer_path(columns, steps):
     """The attention layer behind the reference's class interface (include/sentinel_hip/HipCausalSelfAttention.hpp:
     projections, rotation, attention core, output projection and their backward) with flash attention on and off, on
-    the reference's flash-parity shapes: the "attention fwd/bwd ms" of its train profile.  Timed by the C++ program
+    the reference's flash-parity shapes, and with the projection products in mixed precision as well
+    (flash_mixed_projections): the "attention fwd/bwd ms" of its train profile.  Timed by the C++ program
     tests/cpp/bench_layer (the layer is C++), started as a child process before this process touches the GPU."""
     import subprocess
     exe = os.path.join(ROOT, "tests", "cpp", "bench_layer")

@@ -5,7 +5,9 @@
 // members, uploadFrom, forward(input, out, segmentLength) and backward(outputGradient, inputGradient, four weight
 // gradients), so that a transformer block written against the CUDA class can hold this one instead. What it does
 // (Cuda/CudaCausalSelfAttention.cu:181-253 forward, :345-547 backward, flash branch):
-//   Q = Wq X, K = Wk X, V = Wv X        fp32 GEMMs (rocBLAS; the CUDA class uses cuBLASLt)
+//   Q = Wq X, K = Wk X, V = Wv X        fp32 GEMMs (rocBLAS; the CUDA class uses cuBLASLt), or, with
+//                                       HipAmp::preferMixedPrecision, 16-bit operands with fp32 accumulation
+//                                       (CudaAmp::preferMixedPrecision, Cuda/CudaMatmul.cu:413)
 //   RoPE on Q, K, packs restart at position 0 (segmentLength)
 //   flash attention, grouped-query heads read in place (no expandKvHeadsInto / reduceKvHeadGradsInto)
 //   Y = Wo A
@@ -32,6 +34,7 @@
 #ifndef SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
 #define SENTINEL_HIP_HIPCAUSALSELFATTENTION_HPP
 
+#include "HipAmp.hpp"
 #include "HipFlashAttention.hpp"
 
 #include <rocblas/rocblas.h>
@@ -41,7 +44,7 @@
 namespace sentinel_hip_host {
 
 /// C = op(A) op(B) (+ C) on row-major fp32 device matrices; stands for CudaMatrix::multiplyInto and its
-/// transposed variants (sentinel/NeuralNet/Cuda/CudaMatmul.hpp).
+/// transposed variants (sentinel/NeuralNet/Cuda/CudaMatmul.hpp), including its mixed-precision branch (HipAmp).
 class HipGemm {
 public:
     static void multiplyInto(const HipMatrix& a, const HipMatrix& b, HipMatrix& c, bool transposeA = false,
@@ -61,6 +64,11 @@ public:
         rocblas_handle h = handle();
         if (rocblas_set_stream(h, HipFlashAttention::activeStream()) != rocblas_status_success)
             throw std::runtime_error("HipGemm rocblas_set_stream failed");
+        // mixed precision first, as CudaMatrix::multiplyInto does (Cuda/CudaMatmul.cu:413): 16-bit copies of both
+        // operands, fp32 accumulation; products too small for it and a switched-off HipAmp fall through to fp32
+        if (HipAmp::tryMultiply(h, a.buffer.deviceData, a.elementCount(), a.cols, transposeA, b.buffer.deviceData,
+                                b.elementCount(), b.cols, transposeB, c.buffer.deviceData, n, m, n, ka, accumulate))
+            return;
         // row-major C = op(A) op(B)  <=>  column-major C^T = op(B)^T op(A)^T, each row-major matrix read as its transpose
         const rocblas_status st = rocblas_sgemm(
             h, transposeB ? rocblas_operation_transpose : rocblas_operation_none,
@@ -171,6 +179,45 @@ private:
     }
 };
 
+/// A layer's weights as HipAmp knows them (CudaAmp::registerMasterWeight calls of the CUDA class,
+/// Cuda/CudaCausalSelfAttention.cu:146-151, :164-172). The registrations end with this object, so that no other
+/// allocation at a dead weight's address can be served its 16-bit copy.
+class MasterWeightRegistrations {
+public:
+    MasterWeightRegistrations() = default;
+    MasterWeightRegistrations(const MasterWeightRegistrations&) = delete;
+    MasterWeightRegistrations& operator=(const MasterWeightRegistrations&) = delete;
+    MasterWeightRegistrations(MasterWeightRegistrations&& other) noexcept : pointers(std::move(other.pointers)) {
+        other.pointers.clear();
+    }
+    MasterWeightRegistrations& operator=(MasterWeightRegistrations&& other) noexcept {
+        if (this != &other) {
+            clear();
+            pointers = std::move(other.pointers);
+            other.pointers.clear();
+        }
+        return *this;
+    }
+    ~MasterWeightRegistrations() { clear(); }
+
+    /// register exactly these matrices (empty ones are skipped); earlier registrations of this object end
+    void set(std::initializer_list<const HipMatrix*> weights) {
+        clear();
+        for (const HipMatrix* weight : weights) {
+            if (weight == nullptr || weight->empty()) continue;
+            HipAmp::registerMasterWeight(weight->buffer.deviceData, weight->elementCount());
+            pointers.push_back(weight->buffer.deviceData);
+        }
+    }
+    void clear() {
+        for (const float* pointer : pointers) HipAmp::forgetMasterWeight(pointer);
+        pointers.clear();
+    }
+
+private:
+    std::vector<const float*> pointers;
+};
+
 class HipCausalSelfAttention {
 public:
     HipMatrix queryWeight, keyWeight, valueWeight, outputWeight;
@@ -178,6 +225,9 @@ public:
     /// matrices above and below are then views of their row blocks
     HipMatrix qkvWeight, qkvProjected, qkvGradient, qkvWeightGradient;
     HipMatrix cosTable, sinTable;
+    /// the matrices the projection products read, registered with HipAmp: their 16-bit copies are kept until
+    /// HipAmp::invalidateMasterWeightHalves() (call it after every optimizer step when preferMixedPrecision is on)
+    MasterWeightRegistrations masterWeights;
     int headCount = 0;
     int kvHeadCount = 0;
     int headDimension = 0;
@@ -252,6 +302,16 @@ public:
             }
         cosTable.upload(cosHost, static_cast<size_t>(maximumPositionCount), static_cast<size_t>(pairCount));
         sinTable.upload(sinHost, static_cast<size_t>(maximumPositionCount), static_cast<size_t>(pairCount));
+        registerMasterWeights();
+    }
+
+    /// (re-)register the weights the products read: the stacked matrix of a multi-head layer, else the three split ones,
+    /// and the output weight. Registering marks their 16-bit copies stale (CudaAmp::registerMasterWeight).
+    void registerMasterWeights() {
+        if (usesFusedQkv() && !qkvWeight.empty())
+            masterWeights.set({&qkvWeight, &outputWeight});
+        else
+            masterWeights.set({&queryWeight, &keyWeight, &valueWeight, &outputWeight});
     }
 
     static HipCausalSelfAttention createFrom(const HostAttentionWeights& host) {
@@ -268,7 +328,10 @@ public:
     /// there is nothing to copy; only split weights that were replaced by matrices of their own are stacked again.
     void syncFusedQkvWeight() {
         if (!usesFusedQkv()) {
-            qkvWeight = HipMatrix();
+            if (!qkvWeight.empty()) {
+                qkvWeight = HipMatrix();
+                registerMasterWeights();
+            }
             return;
         }
         if (queryWeight.empty() || keyWeight.empty() || valueWeight.empty()) return;
@@ -292,6 +355,7 @@ public:
         throwIfHipFailed(hipStreamSynchronize(HipFlashAttention::activeStream()), "HipCausalSelfAttention::syncFusedQkvWeight");
         qkvWeight = std::move(fresh);
         for (int i = 0; i < 3; ++i) parts[i]->viewRows(qkvWeight, i * rows, rows);
+        registerMasterWeights();
     }
 
     /// release dense-only scratch (CudaCausalSelfAttention::releaseDenseAttentionScratch, :59-77)
@@ -340,6 +404,7 @@ public:
         activeSegmentLength = segmentLength;
         activePackCount = columns / segmentLength;
         usedFlashAttention = canUseFlashAttention(segmentLength);
+        const HipAmp::ActivationCastScope castOnce;  // no cast buffer below is rewritten once a product has read it
 
         inputCache.ensureSize(input.rows, input.cols);
         throwIfHipFailed(hipMemcpyAsync(inputCache.buffer.deviceData, input.buffer.deviceData, input.byteCount(),
@@ -394,6 +459,8 @@ public:
         } else if (probabilities.rows != static_cast<size_t>(headCount) * activePackCount) {
             throw std::invalid_argument(std::string(op) + " head cache size mismatch");
         }
+        // outputGradient, the stacked / split projection gradients and inputCache feed two or three products each
+        const HipAmp::ActivationCastScope castOnce;
         HipGemm::multiplyInto(outputGradient, attended, outputWeightGradient, false, true);
         HipGemm::multiplyInto(outputWeight, outputGradient, attendedGradient, true, false);
         if (usesFusedQkv()) {

@@ -140,6 +140,17 @@ SENTINEL_HIP_API int sentinel_hip_rope_rotate(float* tensor, int heads, int head
                              const float* sin_table, int table_positions, int inverse, void* stream);
 
 /*
+ * destination[i] = source[i] rounded to nearest even in `dtype` (SENTINEL_HIP_BF16 or SENTINEL_HIP_F16), for
+ * element_count fp32 values in device memory; fp16 values beyond its range become infinities. The operand cast of the
+ * layer's mixed-precision projection GEMMs: replaces CudaAmp::castFloatBufferToHalf (Cuda/CudaAmp.hpp:83,
+ * Cuda/CudaAmp.cu:467-473, :523-527), which CudaMatrix::multiplyInto runs on both operands when
+ * CudaAmp::preferMixedPrecision is set (Cuda/CudaMatmul.cu:413, Cuda/CudaAmp.cu:892-918). source must be 4-byte and
+ * destination 2-byte aligned (16-byte aligned buffers take the wide path); element_count 0 is a no-op.
+ */
+SENTINEL_HIP_API int sentinel_hip_cast_to_16bit(const float* source, void* destination, size_t element_count, int dtype,
+                               void* stream);
+
+/*
  * sentinel_hip_flash_fwd / _bwd on UNROTATED q and k: token t of every pack is rotated with table row
  * position_offset + t on the way into the kernels, and dq, dk come back rotated back (gradients with respect
  * to the unrotated tensors). One call replaces the sequence the CUDA layer runs around the attention core:

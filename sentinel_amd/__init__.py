@@ -1,5 +1,6 @@
 """MI355X-native causal flash attention behind Sentinel's CudaFlashAttention interface."""
 from .flash_attention import (  # noqa: F401
+    HipAmp,
     HipFlashAttention,
     HipOps,
     collect_kernel_timings,

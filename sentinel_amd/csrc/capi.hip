@@ -531,6 +531,22 @@ extern "C" int sentinel_hip_rope_rotate(float* tensor, int heads, int head_dim, 
     return SENTINEL_HIP_OK;
 }
 
+extern "C" int sentinel_hip_cast_to_16bit(const float* source, void* destination, size_t element_count, int dtype,
+                                          void* stream_ptr) {
+    const char* op = "sentinel_hip_cast_to_16bit";
+    if (dtype != SENTINEL_HIP_BF16 && dtype != SENTINEL_HIP_F16)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s dtype must be SENTINEL_HIP_BF16 or SENTINEL_HIP_F16", op);
+    if (element_count == 0) return SENTINEL_HIP_OK;
+    if (!source || !destination) return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s empty buffer", op);
+    if (reinterpret_cast<uintptr_t>(source) % 4 != 0 || reinterpret_cast<uintptr_t>(destination) % 2 != 0)
+        return fail(SENTINEL_HIP_INVALID_ARGUMENT, "%s misaligned buffer", op);
+    if (!sentinel_hip_device_available()) return fail(SENTINEL_HIP_RUNTIME, "%s no HIP device", op);
+    const hipError_t err = launch_cast_f32_to_16bit(static_cast<Elem>(dtype), source, destination, element_count,
+                                                    static_cast<hipStream_t>(stream_ptr));
+    if (err != hipSuccess) return fail_hip("cast launch", err);
+    return SENTINEL_HIP_OK;
+}
+
 namespace {
 
 // argument checks shared by the dense path's two softmax entry points; messages follow

@@ -120,6 +120,8 @@ hipError_t launch_columns_to_bhtd(Elem type, const float* src, void* dst, int he
                                   int seq_len, int packs, RopeTables rope, hipStream_t stream, int padded_dim = 0);
 hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int heads, int head_dim, int stride_columns,
                                   int seq_len, int packs, RopeTables inverse_rope, hipStream_t stream, int padded_dim = 0);
+// flat cast of `count` fp32 values to bf16 / fp16, round to nearest even (operands of the layer's mixed-precision GEMMs)
+hipError_t launch_cast_f32_to_16bit(Elem type, const float* src, void* dst, size_t count, hipStream_t stream);
 // single-query attention against the K/V cache (fp32 column layout, `stride` positions per row, `length` used)
 size_t decode_workspace_bytes(int q_heads, int head_dim, int length);
 // window / global_tokens: the layer's sparse mask for the query at position length - 1 (window <= 0: none)

@@ -184,6 +184,30 @@ __global__ __launch_bounds__(256) void rope_rotate_f32_kernel(float* __restrict_
     even_at[stride] = odd;
 }
 
+// Flat fp32 -> 16-bit cast (round to nearest even; fp16 values beyond its range become infinities, like the conversion
+// instruction gives them): the operands of the layer's mixed-precision projection GEMMs.  WIDE: both pointers 16-byte
+// aligned, eight values per thread and trip (two 16-byte loads, one 16-byte store); the count's last values, fewer than
+// eight, go one per thread through the first workgroup.
+template <typename E, bool WIDE>
+__global__ __launch_bounds__(256) void cast_f32_to_16bit_kernel(const float* __restrict__ src,
+                                                                 unsigned short* __restrict__ dst, size_t count) {
+    const size_t first = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * 256;
+    if (WIDE) {
+        const size_t groups = count / 8;
+        for (size_t i = first; i < groups; i += step) {
+            const float4 a = reinterpret_cast<const float4*>(src)[2 * i];
+            const float4 b = reinterpret_cast<const float4*>(src)[2 * i + 1];
+            const u32x4 r = {E::pack2(a.x, a.y), E::pack2(a.z, a.w), E::pack2(b.x, b.y), E::pack2(b.z, b.w)};
+            reinterpret_cast<u32x4*>(dst)[i] = r;
+        }
+        const size_t at = groups * 8 + first;
+        if (first < 8 && at < count) dst[at] = (unsigned short)(E::pack2(src[at], 0.0f) & 0xffffu);
+    } else {
+        for (size_t i = first; i < count; i += step) dst[i] = (unsigned short)(E::pack2(src[i], 0.0f) & 0xffffu);
+    }
+}
+
 }  // namespace
 
 hipError_t launch_rope_rotate_f32(float* tensor, int heads, int head_dim, int stride_columns, int columns,
@@ -269,6 +293,26 @@ hipError_t launch_bhtd_to_columns(Elem type, const void* src, float* dst, int he
         if (v4) SENTINEL_LAUNCH(Bf16, true); else SENTINEL_LAUNCH(Bf16, false);
     } else if (type == Elem::F16) {
         if (v4) SENTINEL_LAUNCH(Fp16, true); else SENTINEL_LAUNCH(Fp16, false);
+    } else {
+        return hipErrorInvalidValue;
+    }
+#undef SENTINEL_LAUNCH
+    return hipGetLastError();
+}
+
+hipError_t launch_cast_f32_to_16bit(Elem type, const float* src, void* dst, size_t count, hipStream_t stream) {
+    if (count == 0) return hipSuccess;
+    const bool wide = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
+    const size_t per_thread = wide ? 8 : 1;
+    const size_t wanted = (count + 256 * per_thread - 1) / (256 * per_thread);
+    const dim3 grid((unsigned)(wanted < 8192 ? wanted : 8192));  // grid-stride beyond 16 M values
+    auto out = static_cast<unsigned short*>(dst);
+    KernelTimer timer("cast_f32_to_16bit", stream);
+#define SENTINEL_LAUNCH(E, W) hipLaunchKernelGGL((cast_f32_to_16bit_kernel<E, W>), grid, dim3(256), 0, stream, src, out, count)
+    if (type == Elem::BF16) {
+        if (wide) SENTINEL_LAUNCH(Bf16, true); else SENTINEL_LAUNCH(Bf16, false);
+    } else if (type == Elem::F16) {
+        if (wide) SENTINEL_LAUNCH(Fp16, true); else SENTINEL_LAUNCH(Fp16, false);
     } else {
         return hipErrorInvalidValue;
     }

@@ -62,6 +62,8 @@ def load_library():
     lib.sentinel_hip_flash_bwd_sparse.restype = i
     lib.sentinel_hip_rope_rotate.argtypes = [vp] + [i] * 7 + [vp, vp, i, i, vp]
     lib.sentinel_hip_rope_rotate.restype = i
+    lib.sentinel_hip_cast_to_16bit.argtypes = [vp, vp, sz, i, vp]
+    lib.sentinel_hip_cast_to_16bit.restype = i
     ll = ctypes.c_longlong
     lib.sentinel_hip_dense_softmax_fwd.argtypes = [vp, i, ll] + [i] * 6 + [f, vp]
     lib.sentinel_hip_dense_softmax_fwd.restype = i
@@ -249,6 +251,26 @@ class HipOps:
         """CudaOps::rotaryRotateInverseInPlace."""
         return HipOps.rotary_rotate_in_place(tensor, head_count, head_dimension, pair_count, cos_table, sin_table,
                                              position_offset, segment_length, inverse=True, stream=stream)
+
+
+class HipAmp:
+    """The operand cast of the layer's mixed-precision projection GEMMs (class CudaAmp, Cuda/CudaAmp.hpp:54-190)."""
+
+    @staticmethod
+    def cast_to_half(source, dtype=torch.float16, out=None, *, stream=None):
+        """CudaAmp::castFloatBufferToHalf (Cuda/CudaAmp.cu:523-527): `source` (contiguous fp32) rounded to nearest even
+        into a float16 (the reference's type) or bfloat16 tensor of the same shape."""
+        name = "HipAmp::castToHalf"
+        if source is None or source.dtype != torch.float32 or not source.is_contiguous() or not source.is_cuda:
+            raise ValueError(f"{name} expects a contiguous fp32 device tensor")
+        if dtype not in (torch.float16, torch.bfloat16):
+            raise ValueError(f"{name} dtype must be torch.float16 or torch.bfloat16")
+        if out is None:
+            out = torch.empty(source.shape, dtype=dtype, device=source.device)
+        _require(out, source.shape, dtype, source.device, f"{name} destination")
+        _check(load_library().sentinel_hip_cast_to_16bit(_ptr(source), _ptr(out), source.numel(), _DTYPE_CODE[dtype],
+                                                         _stream_handle(stream)))
+        return out
 
 
 class HipFlashAttention:

@@ -4,6 +4,9 @@
 // attention.forward(input, attended, sequenceLength) and attention.backward(gradient, inputGradient, four weight
 // gradients), averaged over the timed steps.  Shapes are the reference's flash-parity ones (main.cpp:640-643:
 // (E, H, T) = (768,12,128), (768,12,256), (768,12,1024)), packed to `columns` tokens per step like its packed batches.
+// A third timing has the projection products in mixed precision as well (HipAmp::preferMixedPrecision, fp16 operands,
+// the reference's CudaAmp::preferMixedPrecision); the weights' 16-bit copies are kept across steps, as between two
+// optimizer steps.
 //
 //   bench_layer [columns=4096] [steps=20] [warmup=3]
 // prints one JSON object on stdout; bench.py --layer-path runs it and puts that object into its line.
@@ -31,7 +34,7 @@ struct Timing {
     float backwardMs = 0.0f;
 };
 
-static Timing timeLayer(int e, int heads, int T, int packs, bool preferFlash, int steps, int warmup) {
+static Timing timeLayer(int e, int heads, int T, int packs, bool preferFlash, bool mixedProjections, int steps, int warmup) {
     const int d = e / heads, cols = packs * T;
     unsigned state = 271u;
     const float bound = 1.0f / std::sqrt(static_cast<float>(e));
@@ -45,6 +48,8 @@ static Timing timeLayer(int e, int heads, int T, int packs, bool preferFlash, in
     host.kvHeadCount = heads;
     host.headDimension = d;
     host.maximumPositionCount = T;
+    HipAmp::preferMixedPrecision() = mixedProjections;
+    const unsigned long long mixedBefore = HipAmp::mixedProductCount();
     HipCausalSelfAttention layer = HipCausalSelfAttention::createFrom(host);
     layer.preferFlashAttention = preferFlash;
 
@@ -72,6 +77,9 @@ static Timing timeLayer(int e, int heads, int T, int packs, bool preferFlash, in
         sum.backwardMs += b;
     }
     for (hipEvent_t& m : marks) throwIfHipFailed(hipEventDestroy(m), "hipEventDestroy");
+    HipAmp::preferMixedPrecision() = false;
+    if ((HipAmp::mixedProductCount() != mixedBefore) != mixedProjections)
+        throw std::logic_error("bench_layer: unexpected projection arithmetic");
     sum.forwardMs /= static_cast<float>(steps);
     sum.backwardMs /= static_cast<float>(steps);
     return sum;
@@ -88,21 +96,26 @@ int main(int argc, char** argv) {
     try {
         HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_BF16;
         const int shapes[3][3] = {{768, 12, 128}, {768, 12, 256}, {768, 12, 1024}};
-        std::string json = "{\"compute\": \"bf16 attention arithmetic, fp32 projections (rocBLAS)\", \"columns_per_step\": " +
+        std::string json = "{\"compute\": \"bf16 attention arithmetic; projections fp32 (rocBLAS sgemm) in flash / dense, fp16 operands with "
+                           "fp32 accumulation (rocblas_gemm_ex) in flash_mixed_projections\", \"columns_per_step\": " +
                            std::to_string(columns) + ", \"steps\": " + std::to_string(steps) + ", \"shapes\": [";
         for (int i = 0; i < 3; ++i) {
             const int e = shapes[i][0], heads = shapes[i][1], T = shapes[i][2];
             const int packs = columns / T > 0 ? columns / T : 1;
-            const Timing flash = timeLayer(e, heads, T, packs, true, steps, warmup);
-            const Timing dense = timeLayer(e, heads, T, packs, false, steps, warmup);
-            char row[512];
+            const Timing flash = timeLayer(e, heads, T, packs, true, false, steps, warmup);
+            const Timing dense = timeLayer(e, heads, T, packs, false, false, steps, warmup);
+            const Timing mixed = timeLayer(e, heads, T, packs, true, true, steps, warmup);
+            char row[768];
             std::snprintf(row, sizeof row,
                           "%s{\"embedding_dim\": %d, \"heads\": %d, \"seq_len\": %d, \"packs\": %d, "
                           "\"flash\": {\"attention_fwd_ms\": %.4f, \"attention_bwd_ms\": %.4f}, "
                           "\"dense\": {\"attention_fwd_ms\": %.4f, \"attention_bwd_ms\": %.4f}, "
-                          "\"tokens_per_s_flash\": %.0f, \"tokens_per_s_dense\": %.0f}",
+                          "\"flash_mixed_projections\": {\"attention_fwd_ms\": %.4f, \"attention_bwd_ms\": %.4f}, "
+                          "\"tokens_per_s_flash\": %.0f, \"tokens_per_s_dense\": %.0f, \"tokens_per_s_flash_mixed_projections\": %.0f}",
                           i ? ", " : "", e, heads, T, packs, flash.forwardMs, flash.backwardMs, dense.forwardMs, dense.backwardMs,
-                          packs * T / ((flash.forwardMs + flash.backwardMs) * 1e-3), packs * T / ((dense.forwardMs + dense.backwardMs) * 1e-3));
+                          mixed.forwardMs, mixed.backwardMs, packs * T / ((flash.forwardMs + flash.backwardMs) * 1e-3),
+                          packs * T / ((dense.forwardMs + dense.backwardMs) * 1e-3),
+                          packs * T / ((mixed.forwardMs + mixed.backwardMs) * 1e-3));
             json += row;
         }
         json += "]}";

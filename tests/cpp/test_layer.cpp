@@ -11,6 +11,7 @@
 #include <cmath>
 #include <cstdio>
 #include <stdexcept>
+#include <string>
 #include <vector>
 
 using namespace sentinel_hip_host;
@@ -230,6 +231,90 @@ static void runGeneration(const char* name, int e, int heads, int kvHeads, int d
     if (cache.length != prompt) throw std::runtime_error("prefill did not reset the cache");
 }
 
+// HipAmp::preferMixedPrecision (CudaAmp::preferMixedPrecision): the projection products through 16-bit operand copies
+// with fp32 accumulation, against the same fp32 oracle layer; which path ran is read from HipAmp::mixedProductCount.
+static void runMixedPrecision() {
+    struct Restore {
+        ~Restore() {
+            HipAmp::preferMixedPrecision() = false;
+            HipAmp::operandType() = SENTINEL_HIP_F16;
+            HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
+        }
+    } restore;
+    HipAmp::preferMixedPrecision() = true;
+    const int types[2] = {SENTINEL_HIP_F16, SENTINEL_HIP_BF16};
+    for (int type : types) {
+        HipAmp::operandType() = type;
+        const char* tag = type == SENTINEL_HIP_F16 ? "fp16" : "bf16";
+        unsigned long long before = HipAmp::mixedProductCount();
+        runCase((std::string("amp ") + tag + " GEMMs, bf16 attention E256 H4 d64 T128 packs2").c_str(), 256, 4, 4, 64, 128, 2,
+                SENTINEL_HIP_COMPUTE_BF16, 2e-2f);
+        if (HipAmp::mixedProductCount() < before + 6) throw std::runtime_error("stacked-QKV layer: the 16-bit products did not run");
+        before = HipAmp::mixedProductCount();
+        runCase((std::string("amp ") + tag + " GEMMs, fp16 attention GQA 4q/1kv d128 T256").c_str(), 256, 4, 1, 128, 256, 1,
+                SENTINEL_HIP_COMPUTE_F16, 2e-2f);
+        if (HipAmp::mixedProductCount() < before + 12) throw std::runtime_error("grouped-query layer: the 16-bit products did not run");
+        runCase((std::string("amp ") + tag + " GEMMs, fp32 attention E256 H8 d32 T96 packs3").c_str(), 256, 8, 8, 32, 96, 3,
+                SENTINEL_HIP_COMPUTE_AUTO, 2e-2f);
+        runCase((std::string("amp ") + tag + " GEMMs, dense attention E256 H4 d64 T128 packs2").c_str(), 256, 4, 4, 64, 128, 2,
+                SENTINEL_HIP_COMPUTE_AUTO, 2e-2f, 0, 0, false);
+    }
+    HipAmp::operandType() = SENTINEL_HIP_F16;
+    // products below the reference's size rule (contraction < 256) stay fp32: same bits as with the switch off
+    {
+        const unsigned long long before = HipAmp::mixedProductCount();
+        runCase("amp on, E64: products too small, fp32", 64, 4, 4, 16, 48, 1, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f);
+        if (HipAmp::mixedProductCount() != before) throw std::runtime_error("a product below the size rule took the 16-bit path");
+    }
+    // master weights: the 16-bit copy is kept until invalidateMasterWeightHalves, registrations follow the layer
+    const int e = 256, heads = 4, d = 64, T = 64;
+    unsigned state = 77u;
+    HostAttentionWeights host;
+    host.embeddingDim = e;
+    host.headCount = heads;
+    host.headDimension = d;
+    host.maximumPositionCount = T;
+    const float bound = 1.0f / std::sqrt(static_cast<float>(e));
+    host.queryWeight = lcg(static_cast<size_t>(e) * e, state, bound);
+    host.keyWeight = lcg(static_cast<size_t>(e) * e, state, bound);
+    host.valueWeight = lcg(static_cast<size_t>(e) * e, state, bound);
+    host.outputWeight = lcg(static_cast<size_t>(e) * e, state, bound);
+    HipMatrix x, y1, y2, y3, y4;
+    x.upload(lcg(static_cast<size_t>(e) * T, state, 1.0f), e, T);
+    const float* deadWeight = nullptr;
+    size_t deadCount = 0;
+    {
+        HipCausalSelfAttention built = HipCausalSelfAttention::createFrom(host);
+        HipCausalSelfAttention layer = std::move(built);  // registrations move with the buffers
+        layer.forward(x, y1, T);
+        deadWeight = layer.outputWeight.buffer.deviceData;
+        deadCount = layer.outputWeight.elementCount();
+        if (HipAmp::masterWeightHalfOrNull(deadWeight, deadCount, SENTINEL_HIP_F16) == nullptr ||
+            HipAmp::masterWeightHalfOrNull(layer.qkvWeight.buffer.deviceData, layer.qkvWeight.elementCount(), SENTINEL_HIP_F16) == nullptr)
+            throw std::runtime_error("the layer's weights are not registered with HipAmp");
+        // the optimizer's step: new output weights in the same buffer
+        layer.outputWeight.upload(lcg(static_cast<size_t>(e) * e, state, bound), e, e);
+        if (layer.outputWeight.buffer.deviceData != deadWeight) throw std::runtime_error("upload moved the weight");
+        layer.forward(x, y2, T);  // the kept copy still serves: the caller has not said that the weights changed
+        if (y2.download() != y1.download()) throw std::runtime_error("the kept 16-bit weight copy was not used");
+        HipAmp::invalidateMasterWeightHalves();
+        layer.forward(x, y3, T);
+        HipAmp::preferMixedPrecision() = false;
+        layer.forward(x, y4, T);
+        HipAmp::preferMixedPrecision() = true;
+        const float fresh = relErr(y3.download(), y4.download()), stale = relErr(y1.download(), y4.download());
+        std::printf("  %-40s  new weights: %.2e from fp32, old copy: %.2e\n", "amp master weight copies", fresh, stale);
+        if (fresh > 2e-2f || stale < 0.1f) throw std::runtime_error("invalidateMasterWeightHalves did not refresh the copy");
+    }
+    if (HipAmp::masterWeightHalfOrNull(deadWeight, deadCount, SENTINEL_HIP_F16) != nullptr)
+        throw std::runtime_error("a dead layer's weight is still registered with HipAmp");
+    expectThrow("operand type", [&] {
+        HipAmp::operandType() = SENTINEL_HIP_F32;
+        HipCausalSelfAttention layer = HipCausalSelfAttention::createFrom(host);
+        layer.forward(x, y1, T);
+    });
+}
+
 int main() {
     try {
         if (!sentinel_hip_device_available()) {
@@ -274,6 +359,7 @@ int main() {
         runGeneration("generate dense prefill H4 d16 32+32", 64, 4, 4, 16, 32, 64, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 0, 0, false);
         runGeneration("generate dense prefill sparse GQA W9 G2", 64, 4, 2, 16, 20, 60, SENTINEL_HIP_COMPUTE_AUTO, 1e-4f, 9, 2, false);
         HipFlashAttention::computeType() = SENTINEL_HIP_COMPUTE_AUTO;
+        runMixedPrecision();
 
         // configurations this layer does not run are refused, not approximated
         HostAttentionWeights host;
