@@ -13,7 +13,9 @@
 //  * activations are cast again for every product unless the caller opens an ActivationCastScope: the reference keeps
 //    four casts keyed by source address alone (getOrCastActivationHalf, Cuda/CudaAmp.cu:55-79), which a buffer
 //    rewritten in place defeats; inside a scope (the layer opens one per forward / backward call, during which no
-//    cast buffer is rewritten) a tensor that feeds several products is cast once;
+//    cast buffer is rewritten) a tensor that feeds several products is cast once, and the layer keeps the 16-bit copies
+//    of its input and of the attended matrix from the forward call for the backward call's weight-gradient products
+//    (persistActivationHalf, as the reference does for its cached inputs, Cuda/CudaAmp.cu:862-869);
 //  * forgetMasterWeight(): a layer that dies takes its registrations with it, so that another allocation at the same
 //    address can never be served a dead weight's copy;
 //  * products that accumulate into the result (beta = 1) take the 16-bit path too.
@@ -46,6 +48,12 @@ public:
 
     /// products that took the 16-bit path since the process started (tests and benches read it to see which path ran)
     static unsigned long long& mixedProductCount() {
+        static unsigned long long value = 0;
+        return value;
+    }
+
+    /// operand casts launched since the process started (weights and activations)
+    static unsigned long long& castCount() {
         static unsigned long long value = 0;
         return value;
     }
@@ -96,15 +104,40 @@ public:
     public:
         ActivationCastScope() {
             clearActivationSlots();
+            adoptedCopies().clear();
             scopeOpen() = true;
         }
         ~ActivationCastScope() {
             scopeOpen() = false;
             clearActivationSlots();
+            adoptedCopies().clear();
         }
         ActivationCastScope(const ActivationCastScope&) = delete;
         ActivationCastScope& operator=(const ActivationCastScope&) = delete;
+
+        /// until the scope ends, products that read `source` (elementCount fp32 values) take this 16-bit copy of it, which
+        /// the caller made (persistActivationHalf) and keeps alive and current
+        void adopt(const float* source, size_t elementCount, const void* half, int type) {
+            if (source == nullptr || half == nullptr || elementCount == 0) return;
+            adoptedCopies().push_back(AdoptedCopy{source, elementCount, half, type});
+        }
     };
+
+    /// CudaAmp::persistActivationHalf (Cuda/CudaAmp.cu:862-869): a 16-bit copy of an activation in a buffer of the
+    /// caller's, e.g. kept from the forward call for the weight-gradient products of the backward call; returns the type
+    /// it was cast to (operandType() at the time)
+    static int persistActivationHalf(const float* source, size_t elementCount, HipDeviceBuffer& destination) {
+        const int type = operandType();
+        if (type != SENTINEL_HIP_F16 && type != SENTINEL_HIP_BF16)
+            throw std::invalid_argument("HipAmp::operandType must be SENTINEL_HIP_F16 or SENTINEL_HIP_BF16");
+        cast(source, elementCount, type, destination);
+        return type;
+    }
+
+    /// the size rule of tryMultiply (CudaAmp::launchCublasLtMatmulFp16, Cuda/CudaAmp.cu:896) and the switch
+    static bool wouldMultiplyMixed(size_t m, size_t n, size_t k) {
+        return preferMixedPrecision() && k >= 256 && m >= 32 && n >= 32;
+    }
 
     /// C (+)= op(A) op(B) on row-major fp32 matrices through 16-bit copies of A and B; false (nothing done) when the
     /// switch is off or the product is too small for it, the caller then multiplies in fp32. lda / ldb / ldc: floats
@@ -112,8 +145,7 @@ public:
     static bool tryMultiply(rocblas_handle handle, const float* a, size_t aElements, size_t lda, bool transposeA, const float* b,
                             size_t bElements, size_t ldb, bool transposeB, float* c, size_t ldc, size_t m, size_t n, size_t k,
                             bool accumulate) {
-        if (!preferMixedPrecision()) return false;
-        if (k < 256 || m < 32 || n < 32) return false;  // CudaAmp::launchCublasLtMatmulFp16's rule
+        if (!wouldMultiplyMixed(m, n, k)) return false;
         const int type = operandType();
         if (type != SENTINEL_HIP_F16 && type != SENTINEL_HIP_BF16)
             throw std::invalid_argument("HipAmp::operandType must be SENTINEL_HIP_F16 or SENTINEL_HIP_BF16");
@@ -166,6 +198,16 @@ private:
         unsigned long long lastUsed = 0;
     };
     static constexpr int activationSlotCount = 4;
+    struct AdoptedCopy {
+        const float* source;
+        size_t elementCount;
+        const void* half;
+        int type;
+    };
+    static std::vector<AdoptedCopy>& adoptedCopies() {
+        static std::vector<AdoptedCopy>* all = new std::vector<AdoptedCopy>();
+        return *all;
+    }
 
     static std::vector<MasterWeightHalf>& masterWeights() {
         // never destroyed: objects that forget their registrations in their destructors may outlive any static
@@ -190,6 +232,7 @@ private:
     }
 
     static void cast(const float* source, size_t elementCount, int type, HipDeviceBuffer& destination) {
+        ++castCount();
         destination.ensureCapacity(elementCount * 2);
         const int code = sentinel_hip_cast_to_16bit(source, destination.deviceData, elementCount, type,
                                                     HipFlashAttention::activeStream());
@@ -204,6 +247,8 @@ private:
     /// run in order, so a slot can be filled again as soon as the product that read it has been launched.
     static const void* operand16(const float* source, size_t elementCount, int type) {
         if (const void* weight = masterWeightHalfOrNull(source, elementCount, type)) return weight;
+        for (const AdoptedCopy& copy : adoptedCopies())
+            if (copy.source == source && copy.elementCount == elementCount && copy.type == type) return copy.half;
         static unsigned long long useCounter = 1;
         ActivationSlot* slots = activationSlots();
         if (scopeOpen())

@@ -243,6 +243,10 @@ public:
     HipMatrix query, key, value, attended, output;
     HipMatrix inputCache, attendedGradient, queryGradient, keyGradient, valueGradient;
     HipMatrix flashLogSumExp, flashDelta;
+    /// mixed-precision projections: the 16-bit copies of the input and of the attended matrix that the forward call's
+    /// products read, kept for the weight-gradient products of the backward call (2 bytes per element of each)
+    HipDeviceBuffer inputHalf, attendedHalf;
+    int keptHalfType = -1;  // SENTINEL_HIP_F16 / _BF16 while both copies match inputCache and attended, else -1
     /// the forward call's 16-bit operands, kept for the backward call like flashLogSumExp (MFMA arithmetic only; costs
     /// 4 bytes per element of query / key / value in device memory per layer; set keepFlashOperands = false to convert
     /// them again in the backward call instead)
@@ -376,6 +380,9 @@ public:
         HipMatrix* all[] = {&query, &key, &value, &queryGradient, &keyGradient, &valueGradient, &qkvProjected, &qkvGradient,
                             &attended, &output, &inputCache, &attendedGradient};
         for (HipMatrix* m : all) *m = HipMatrix();
+        inputHalf.free();
+        attendedHalf.free();
+        keptHalfType = -1;
     }
 
     /// CudaCausalSelfAttention::canUseFlashAttention (Cuda/CudaCausalSelfAttention.cu:46-57) without the
@@ -404,7 +411,14 @@ public:
         activeSegmentLength = segmentLength;
         activePackCount = columns / segmentLength;
         usedFlashAttention = canUseFlashAttention(segmentLength);
-        const HipAmp::ActivationCastScope castOnce;  // no cast buffer below is rewritten once a product has read it
+        HipAmp::ActivationCastScope castOnce;  // no cast buffer below is rewritten once a product has read it
+        keptHalfType = -1;
+        const bool keepHalves = HipAmp::wouldMultiplyMixed(queryWeight.rows, input.cols, input.rows) &&
+                                HipAmp::wouldMultiplyMixed(outputWeight.rows, input.cols, outputWeight.cols);
+        if (keepHalves) {
+            const int type = HipAmp::persistActivationHalf(input.buffer.deviceData, input.elementCount(), inputHalf);
+            castOnce.adopt(input.buffer.deviceData, input.elementCount(), inputHalf.deviceData, type);
+        }
 
         inputCache.ensureSize(input.rows, input.cols);
         throwIfHipFailed(hipMemcpyAsync(inputCache.buffer.deviceData, input.buffer.deviceData, input.byteCount(),
@@ -440,6 +454,10 @@ public:
                 HipFlashAttention::forwardMultiHead(query, key, value, attended, flashLogSumExp, headCount, headDimension, scale,
                                                     true, 0, segmentLength, activePackCount, kvHeadCount, keptOperands());
         }
+        if (keepHalves) {
+            keptHalfType = HipAmp::persistActivationHalf(attended.buffer.deviceData, attended.elementCount(), attendedHalf);
+            castOnce.adopt(attended.buffer.deviceData, attended.elementCount(), attendedHalf.deviceData, keptHalfType);
+        }
         HipGemm::multiplyInto(outputWeight, attended, out);
     }
 
@@ -460,7 +478,11 @@ public:
             throw std::invalid_argument(std::string(op) + " head cache size mismatch");
         }
         // outputGradient, the stacked / split projection gradients and inputCache feed two or three products each
-        const HipAmp::ActivationCastScope castOnce;
+        HipAmp::ActivationCastScope castOnce;
+        if (keptHalfType >= 0) {  // the forward call's 16-bit copies of the input and of the attended matrix
+            castOnce.adopt(inputCache.buffer.deviceData, inputCache.elementCount(), inputHalf.deviceData, keptHalfType);
+            castOnce.adopt(attended.buffer.deviceData, attended.elementCount(), attendedHalf.deviceData, keptHalfType);
+        }
         HipGemm::multiplyInto(outputGradient, attended, outputWeightGradient, false, true);
         HipGemm::multiplyInto(outputWeight, outputGradient, attendedGradient, true, false);
         if (usesFusedQkv()) {
@@ -580,6 +602,7 @@ private:
         // query / key / value get new contents: 16-bit copies of the old ones must not serve a later backward call (the
         // training forward refills them right after this; prefill and decode do not)
         flashOperands.invalidate();
+        keptHalfType = -1;  // likewise the kept 16-bit copies of input and attended; forward() sets it again
         if (usesFusedQkv()) {
             syncFusedQkvWeight();
             HipGemm::multiplyInto(qkvWeight, input, qkvProjected);

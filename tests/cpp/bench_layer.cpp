@@ -8,7 +8,8 @@
 // the reference's CudaAmp::preferMixedPrecision); the weights' 16-bit copies are kept across steps, as between two
 // optimizer steps.
 //
-//   bench_layer [columns=4096] [steps=20] [warmup=3]
+//   bench_layer [columns=4096] [steps=20] [warmup=3] [only=all|flash|dense|flash_mixed_projections] [seq_len=0]
+// (`only`: time one of the three configurations, `seq_len`: one of the three shapes; e.g. under a profiler)
 // prints one JSON object on stdout; bench.py --layer-path runs it and puts that object into its line.
 #include "../../include/sentinel_hip/HipCausalSelfAttention.hpp"
 
@@ -89,8 +90,11 @@ int main(int argc, char** argv) {
     const int columns = argc > 1 ? std::atoi(argv[1]) : 4096;
     const int steps = argc > 2 ? std::atoi(argv[2]) : 20;
     const int warmup = argc > 3 ? std::atoi(argv[3]) : 3;
-    if (columns <= 0 || steps <= 0 || warmup < 0) {
-        std::fprintf(stderr, "usage: bench_layer [columns] [steps] [warmup]\n");
+    const std::string only = argc > 4 ? argv[4] : "all";
+    const int onlyLength = argc > 5 ? std::atoi(argv[5]) : 0;
+    if (columns <= 0 || steps <= 0 || warmup < 0 ||
+        (only != "all" && only != "flash" && only != "dense" && only != "flash_mixed_projections")) {
+        std::fprintf(stderr, "usage: bench_layer [columns] [steps] [warmup] [all|flash|dense|flash_mixed_projections]\n");
         return 2;
     }
     try {
@@ -99,23 +103,25 @@ int main(int argc, char** argv) {
         std::string json = "{\"compute\": \"bf16 attention arithmetic; projections fp32 (rocBLAS sgemm) in flash / dense, fp16 operands with "
                            "fp32 accumulation (rocblas_gemm_ex) in flash_mixed_projections\", \"columns_per_step\": " +
                            std::to_string(columns) + ", \"steps\": " + std::to_string(steps) + ", \"shapes\": [";
+        bool first = true;
         for (int i = 0; i < 3; ++i) {
             const int e = shapes[i][0], heads = shapes[i][1], T = shapes[i][2];
+            if (onlyLength > 0 && T != onlyLength) continue;
             const int packs = columns / T > 0 ? columns / T : 1;
-            const Timing flash = timeLayer(e, heads, T, packs, true, false, steps, warmup);
-            const Timing dense = timeLayer(e, heads, T, packs, false, false, steps, warmup);
-            const Timing mixed = timeLayer(e, heads, T, packs, true, true, steps, warmup);
             char row[768];
-            std::snprintf(row, sizeof row,
-                          "%s{\"embedding_dim\": %d, \"heads\": %d, \"seq_len\": %d, \"packs\": %d, "
-                          "\"flash\": {\"attention_fwd_ms\": %.4f, \"attention_bwd_ms\": %.4f}, "
-                          "\"dense\": {\"attention_fwd_ms\": %.4f, \"attention_bwd_ms\": %.4f}, "
-                          "\"flash_mixed_projections\": {\"attention_fwd_ms\": %.4f, \"attention_bwd_ms\": %.4f}, "
-                          "\"tokens_per_s_flash\": %.0f, \"tokens_per_s_dense\": %.0f, \"tokens_per_s_flash_mixed_projections\": %.0f}",
-                          i ? ", " : "", e, heads, T, packs, flash.forwardMs, flash.backwardMs, dense.forwardMs, dense.backwardMs,
-                          mixed.forwardMs, mixed.backwardMs, packs * T / ((flash.forwardMs + flash.backwardMs) * 1e-3),
-                          packs * T / ((dense.forwardMs + dense.backwardMs) * 1e-3),
-                          packs * T / ((mixed.forwardMs + mixed.backwardMs) * 1e-3));
+            int at = std::snprintf(row, sizeof row, "%s{\"embedding_dim\": %d, \"heads\": %d, \"seq_len\": %d, \"packs\": %d",
+                                   first ? "" : ", ", e, heads, T, packs);
+            first = false;
+            const char* names[3] = {"flash", "dense", "flash_mixed_projections"};
+            for (int mode = 0; mode < 3; ++mode) {
+                if (only != "all" && only != names[mode]) continue;
+                const Timing t = timeLayer(e, heads, T, packs, mode != 1, mode == 2, steps, warmup);
+                at += std::snprintf(row + at, sizeof row - at,
+                                    ", \"%s\": {\"attention_fwd_ms\": %.4f, \"attention_bwd_ms\": %.4f}, \"tokens_per_s_%s\": %.0f",
+                                    names[mode], t.forwardMs, t.backwardMs, names[mode],
+                                    packs * T / ((t.forwardMs + t.backwardMs) * 1e-3));
+            }
+            std::snprintf(row + at, sizeof row - at, "}");
             json += row;
         }
         json += "]}";

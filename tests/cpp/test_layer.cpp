@@ -267,7 +267,7 @@ static void runMixedPrecision() {
         if (HipAmp::mixedProductCount() != before) throw std::runtime_error("a product below the size rule took the 16-bit path");
     }
     // master weights: the 16-bit copy is kept until invalidateMasterWeightHalves, registrations follow the layer
-    const int e = 256, heads = 4, d = 64, T = 64;
+    const int e = 256, heads = 4, d = 64, T = 256;  // every product of the step passes the size rule
     unsigned state = 77u;
     HostAttentionWeights host;
     host.embeddingDim = e;
@@ -299,6 +299,19 @@ static void runMixedPrecision() {
         if (y2.download() != y1.download()) throw std::runtime_error("the kept 16-bit weight copy was not used");
         HipAmp::invalidateMasterWeightHalves();
         layer.forward(x, y3, T);
+        {
+            // a training step with warm weight copies casts four activations: input and attended in the forward call (kept
+            // for the backward call), output gradient and stacked projection gradient in the backward call
+            HipMatrix g, dx, a, b, c, o;
+            g.upload(lcg(static_cast<size_t>(e) * T, state, 1.0f), e, T);
+            const unsigned long long casts = HipAmp::castCount(), products = HipAmp::mixedProductCount();
+            layer.forward(x, y3, T);
+            layer.backward(g, dx, a, b, c, o);
+            if (HipAmp::mixedProductCount() != products + 6 || HipAmp::castCount() != casts + 4)
+                throw std::runtime_error("mixed-precision step: expected 6 products and 4 casts, got " +
+                                         std::to_string(HipAmp::mixedProductCount() - products) + " and " +
+                                         std::to_string(HipAmp::castCount() - casts));
+        }
         HipAmp::preferMixedPrecision() = false;
         layer.forward(x, y4, T);
         HipAmp::preferMixedPrecision() = true;

@@ -34,6 +34,27 @@ def test_cpp_attention_layer_parity_and_exceptions():
     assert "layer ok" in proc.stdout
 
 
+def test_cpp_layer_bench_runs():
+    """tests/cpp/bench_layer (what bench.py's layer_path starts): a short run of every configuration, its JSON parses and
+    the mixed-precision timing really took the 16-bit products (the program checks that itself and fails otherwise)."""
+    import json
+    exe = os.path.join(HERE, "cpp", "bench_layer")
+    assert os.path.exists(exe), "tests/cpp/bench_layer is not built: python -c 'import __graft_entry__ as g; g.build()'"
+    proc = subprocess.run([exe, "512", "2", "1"], capture_output=True, text=True, timeout=110)
+    print(proc.stdout, proc.stderr, flush=True)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    line = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert [s["seq_len"] for s in line["shapes"]] == [128, 256, 1024]
+    for shape in line["shapes"]:
+        for mode in ("flash", "dense", "flash_mixed_projections"):
+            assert shape[mode]["attention_fwd_ms"] > 0 and shape[mode]["attention_bwd_ms"] > 0
+            assert shape["tokens_per_s_" + mode] > 0
+    one = subprocess.run([exe, "512", "2", "1", "flash", "256"], capture_output=True, text=True, timeout=110)
+    assert one.returncode == 0, one.stdout + one.stderr
+    only = json.loads(one.stdout.strip().splitlines()[-1])["shapes"]
+    assert len(only) == 1 and only[0]["seq_len"] == 256 and "dense" not in only[0] and "flash" in only[0]
+
+
 @pytest.mark.parametrize("compute", ["bf16", "fp16"])
 # (q heads, kv heads, head_dim, T, packs, first column, columns behind the window); head dims the kernels have no tiling of
 # their own for (32, 80, 96, 16, 24, 120, 72) are zero-padded to 64 / 128 by the conversion pass
