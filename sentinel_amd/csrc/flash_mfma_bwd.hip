@@ -323,6 +323,8 @@ __global__ __launch_bounds__(kBwdThreads, D <= 64 ? 3 : 2) void dq_mfma_kernel(c
 }
 
 constexpr int kDkvKeyTile = 128;
+// sparse mask without global tokens: windows up to this many keys run the split dK/dV kernel on the persistent grid
+constexpr int kMaxPersistentWindow = 512;
 constexpr int kDkvQueryTile = 64;
 
 // ------------------------------------------------------------------------------------------------
@@ -1073,7 +1075,8 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
         auto launch = [&](auto kernel) {
             static const int resident = resident_workgroups_per_xcd(kernel, kBwdThreads, smem);  // per kernel instantiation
             // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
-            // dispatched in order (long ones first), balances better than a fixed assignment
+            // dispatched in order (long ones first), balances better than a fixed assignment (at head_dim 64 the persistent
+            // grid measured the same for short windows without global tokens and worse for every other mask)
             const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
                                                : plan_persistent_grid(total, k_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dkdv_mfma", stream);
@@ -1098,9 +1101,13 @@ hipError_t run_bwd(const void* q, const void* k, const void* v, const void* out,
                                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
             if (raised != hipSuccess) return raised;
             static const int resident = resident_workgroups_per_xcd(kernel, kDkvSplitThreads, smem);
-            // under the sparse mask the key tiles are short and of two very different lengths: one workgroup per tile,
-            // dispatched in order (long ones first), balances better than a fixed assignment
-            const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
+            // under the sparse mask the key tiles are short and, with global tokens, of two very different lengths: one
+            // workgroup per tile, dispatched in order (long ones first), balances better than a fixed assignment; without
+            // global tokens and with a window of a few stages all tiles are alike and the persistent grid (snake) saves
+            // the workgroup launches (measured at d = 128, T = 4096: window 128 0.267 -> 0.238 ms, window 512
+            // 0.405 -> 0.395 ms, window 2048 0.870 -> 0.925 ms; T = 2048: window 256 0.172 -> 0.152 ms)
+            const bool alike = g.window > 0 && g.window <= kMaxPersistentWindow && g.global_tokens == 0 && tiles_per_xcd > resident;
+            const GridPlan plan = g.window > 0 ? GridPlan{alike ? resident : tiles_per_xcd, 0}
                                                : plan_persistent_grid(total, k_tiles, resident, g.causal != 0, streamed);
             KernelTimer timer("dkdv_mfma", stream);
             hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kDkvSplitThreads), smem, stream, qp, kp, vp, gp, lse, delta, dkp,

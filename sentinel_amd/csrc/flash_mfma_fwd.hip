@@ -314,8 +314,12 @@ hipError_t run_fwd(const void* q, const void* k, const void* v, void* out, float
     auto launch = [&](auto kernel) {
         static const int resident = resident_workgroups_per_xcd(kernel, kFwdThreads, 0);  // per kernel instantiation
         // under the sparse mask tile lengths no longer grow with the tile index, and one workgroup per tile handed out
-        // as slots free up is 6 - 13 % faster than the fixed snake assignment
-        const GridPlan plan = g.window > 0 ? GridPlan{tiles_per_xcd, 0}
+        // as slots free up is 6 - 13 % faster than a fixed assignment; only where a tile is a few trips long (windows up
+        // to two query tiles) the 5 us a workgroup costs to launch weigh more, and the persistent grid, tiles in plain
+        // order, is 5 % faster (measured at d = 128, T = 4096: window 128 0.174 -> 0.166 ms, window 512 0.239 -> 0.249 ms;
+        // T = 2048: window 64 0.085 -> 0.078 ms, window 256 0.109 -> 0.103 ms; no difference at d = 64)
+        const bool short_window = g.window > 0 && g.window <= 2 * kFwdQueryTile && tiles_per_xcd > resident;
+        const GridPlan plan = g.window > 0 ? GridPlan{short_window ? resident : tiles_per_xcd, 0}
                                            : plan_persistent_grid(total, q_tiles, resident, g.causal != 0, streamed);
         KernelTimer timer("fwd_mfma", stream);
         hipLaunchKernelGGL(kernel, dim3(kXcds * plan.slots), dim3(kFwdThreads), 0, stream, qp, kp, vp, op, lse, lm, g, q_tiles,

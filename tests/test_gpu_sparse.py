@@ -117,6 +117,16 @@ def test_mfma_matches_oracle(dtype, shape):
     _bhtd(dtype, shape)
 
 
+@pytest.mark.parametrize("shape", [(8, 8, 128, 1024, 10, 100, 0), (8, 8, 128, 1024, 10, 256, 0), (16, 16, 64, 1024, 12, 70, 0)])
+def test_short_windows_with_more_tiles_than_workgroups_run_at_once(shape):
+    """Short windows without global tokens run the forward (and, at head_dim 128, the dK/dV) kernel on the persistent grid
+    once a die has more tiles than workgroups in flight: 640 query / key tiles at head_dim 128 (80 per die against 64 / 32
+    resident), 1536 query tiles at head_dim 64 (192 per die),
+    so workgroups walk several tiles, the last round is partial, and every tile must still be computed exactly once."""
+    print(f"case sparse persistent {shape}", flush=True)
+    _bhtd("bf16", shape)
+
+
 @pytest.mark.parametrize("d", [128, 96, 32])  # 96 and 32: zero-padded to the kernels' tilings by the conversion pass
 def test_columns_with_mfma_arithmetic_and_fused_rotation(d):
     hq, hkv, t, packs, window, global_tokens = 4, 2, 200, 2, 48, 6
